@@ -1,19 +1,21 @@
 from .schema import (BlockSpec, ConfigError, DeltaRuleSpec, FeedForwardSpec, InputSpec, LatentAttentionSpec,
                      MatrixMemorySpec, MixerSpec, ModelSpec, MoESpec, NormSpec, PairHashSpec, PositionSpec, RunEntry,
-                     SideBySideSpec, StreamAdd, UnknownArchitecture)
+                     ParallelSpec, SideBySideSpec, StreamAdd, UnknownArchitecture, WKVSpec)
 from .registry import (architecture_name, config_from_dict, load_config, register_architecture,
                        registered_architectures)
 from .qwen3 import Qwen3Config
 from .puresun import PuresunConfig
 from .kobolix import KobolixConfig
+from .detatar import DetatarConfig
 
 register_architecture("Qwen3ForCausalLM", Qwen3Config, "qwen3")
 register_architecture("Puresun", PuresunConfig, "puresun")
 register_architecture("Kobolix", KobolixConfig, "kobolix")
+register_architecture("Detatar", DetatarConfig, "detatar")
 
 __all__ = [
     "BlockSpec", "ConfigError", "FeedForwardSpec", "MixerSpec", "ModelSpec", "NormSpec",
     "PositionSpec", "RunEntry", "UnknownArchitecture", "architecture_name", "config_from_dict",
-    "load_config", "register_architecture", "registered_architectures", "Qwen3Config", "PuresunConfig", "KobolixConfig",
+    "load_config", "register_architecture", "registered_architectures", "Qwen3Config", "PuresunConfig", "KobolixConfig", "DetatarConfig", "ParallelSpec", "WKVSpec",
     "InputSpec", "LatentAttentionSpec", "DeltaRuleSpec", "MatrixMemorySpec", "SideBySideSpec", "MoESpec", "PairHashSpec", "StreamAdd",
 ]

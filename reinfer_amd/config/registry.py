@@ -64,4 +64,10 @@ def load_config(model_dir: str):
         if isinstance(gen, dict) and gen.get("eos_token_id") is not None:
             raw = dict(raw)
             raw["eos_token_id"] = gen["eos_token_id"]
-    return config_from_dict(raw)
+    cfg = config_from_dict(raw)
+    if hasattr(cfg, "with_tensor_shapes"):
+        # a design some of whose sizes only the tensors give: the headers of the folder's files are read
+        # (no data), and the configuration takes what it needs from the shapes
+        from ..weights import tensor_shapes
+        cfg = cfg.with_tensor_shapes(tensor_shapes(model_dir))
+    return cfg

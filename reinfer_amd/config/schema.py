@@ -92,6 +92,7 @@ class NormSpec:
     size: int
     eps: float
     offset: float = 0.0  # the stored weight lies around zero: the factor is offset + w (1.0 for "one plus w")
+    groups: int = 1      # the row is normed in this many equal consecutive parts, each over its own root mean square
 
 
 @dataclass(frozen=True)
@@ -144,12 +145,16 @@ class LatentAttentionSpec:
     (``MixerSpec.params`` of the "latent_attention" mixer; heads, scale, window and rotation are the
     ``MixerSpec``'s own fields): a query head is ``head_dim`` unrotated and ``rot_width`` rotated entries, the
     latent ``rank`` wide, a value head ``value_dim``; ``gated``: the concatenated heads are multiplied by the
-    sigmoid of a projection of the mixer's input before the output projection."""
+    sigmoid of a projection of the mixer's input before the output projection, element by element, or, with
+    ``head_gate``, by one number a head. ``q_rank`` > 0: the queries come through a latent of their own,
+    q = W_uq rms(W_dq h) with a plain norm weight (0: q = W_q h)."""
     rank: int
     rot_width: int
     value_dim: int
     norm_eps: float
     gated: bool = True
+    head_gate: bool = False
+    q_rank: int = 0
 
 
 @dataclass(frozen=True)
@@ -161,7 +166,11 @@ class MoESpec:
     logit times ``weight_scale``, not renormalised. ``groups`` > 1: the experts form that many equal runs of
     neighbours, a run's score is the sum of its ``group_top`` largest scores, and only experts of the
     ``groups_kept`` best runs can be chosen. ``shared`` > 0: one more expert of that width, same form, runs
-    for every token with weight 1."""
+    for every token with weight 1, or, with ``shared_gated``, times the sigmoid of one more router output.
+    ``weights`` "softmax": scores are the softmax over all router outputs, the choice is by score plus a stored
+    correction (``correction``) inside the best groups (``group_top`` 1: a group's score is its largest choice
+    score), the weights the chosen scores over their sum + ``norm_eps``. ``identity`` > 0: that many further
+    router outputs behind the experts stand for experts without matrices whose output is their input."""
     experts: int
     top: int
     activation: str = "relu2"
@@ -171,6 +180,10 @@ class MoESpec:
     groups_kept: int = 1
     group_top: int = 2
     shared: int = 0
+    identity: int = 0
+    correction: bool = False
+    norm_eps: float = 0.0
+    shared_gated: bool = False
 
 
 @dataclass(frozen=True)
@@ -185,6 +198,31 @@ class MatrixMemorySpec:
     gate_cap: float
     norm_eps: float
     denom_eps: float = 1e-6
+
+
+@dataclass(frozen=True)
+class WKVSpec:
+    """A matrix state a head with a decay a key channel that depends on the input (``MixerSpec.params`` of the
+    "wkv" mixer): ``heads`` heads of ``dim`` x ``dim``; receptance, key, value, gate and decay each read their own
+    mix of the input row with the row of the token before; the decay's pre-activation goes through a low-rank
+    pair of ``decay_rank``; ``norm_eps`` is the eps of the per-head norm of the read-out."""
+    heads: int
+    dim: int
+    decay_rank: int
+    norm_eps: float
+
+
+@dataclass(frozen=True)
+class ParallelSpec:
+    """Options of the "parallel" arrangement (``BlockSpec.params``). ``token_shift``: what the mixer reads is
+    h + (h' - h) * s with h' the normed row of the token before (zeros for a request's first token, the last row
+    kept in the request's state) and s the vector ``shift_name``. ``gated``: each part's result enters the
+    stream times sigmoid(W h + b), W and b named by ``gate_names`` (mixer, feed-forward; the bias is the name
+    plus ``.b``), h the normed row before any shift."""
+    token_shift: bool = False
+    gated: bool = False
+    shift_name: str = "shift"
+    gate_names: Tuple[str, str] = ("rg1", "rg2")
 
 
 @dataclass(frozen=True)

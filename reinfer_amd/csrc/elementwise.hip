@@ -187,6 +187,62 @@ extern "C" int ra_add_rmsnorm(float* resid, const void* delta, const void* weigh
 }
 
 // ---------------------------------------------------------------------------
+// The same norm in groups: the row is split into `groups` equal consecutive parts, each divided by its own
+// root mean square (eps inside the root), the whole multiplied by w. One workgroup a row, a wave a group at
+// a time (group g goes to wave g mod waves), so a group's sum never leaves its wave.
+// ---------------------------------------------------------------------------
+template <typename TA, typename TW>
+__global__ void add_group_rmsnorm_kernel(float* __restrict__ resid, const TA* __restrict__ delta,
+                                         const TW* __restrict__ w, TA* __restrict__ out,
+                                         const int* __restrict__ rows, int h, int groups, float eps, float dscale) {
+  const int r = blockIdx.x;
+  const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+  float* x = resid + src * h;
+  const TA* dl = delta ? delta + src * h : nullptr;
+  TA* o = out + (size_t)r * h;
+  const int lane = threadIdx.x & (RA_WAVE - 1);
+  const int wave = threadIdx.x / RA_WAVE, waves = blockDim.x / RA_WAVE;
+  const int gs = h / groups;
+  for (int g = wave; g < groups; g += waves) {
+    const int base = g * gs;
+    float ss = 0.f;
+    for (int i = lane; i < gs; i += RA_WAVE) {
+      float v = x[base + i];
+      if (dl) {
+        v += dscale * to_f32(dl[base + i]);
+        if (!rows) x[base + i] = v;      // the same lane reads it back below
+      }
+      ss += v * v;
+    }
+    ss = wave_sum(ss);
+    const float rstd = rsqrtf(ss / (float)gs + eps);
+    for (int i = lane; i < gs; i += RA_WAVE) {
+      float v = x[base + i];
+      if (dl && rows) v += dscale * to_f32(dl[base + i]);
+      o[base + i] = from_f32<TA>(v * rstd * to_f32(w[base + i]));
+    }
+  }
+}
+
+extern "C" int ra_add_group_rmsnorm(float* resid, const void* delta, const void* weight, int weight_dtype,
+                                    void* out, int act_dtype, const int* rows, int n_rows, int hidden, int groups,
+                                    float eps, float delta_scale, hipStream_t stream) {
+  RA_CHECK(n_rows > 0 && hidden > 0, "add_group_rmsnorm: empty input (%d rows, width %d)", n_rows, hidden);
+  RA_CHECK(groups >= 1 && hidden % groups == 0, "add_group_rmsnorm: width %d in %d equal groups", hidden, groups);
+  const int threads = RA_WAVE * (groups >= 8 ? 8 : groups >= 4 ? 4 : groups >= 2 ? 2 : 1);
+#define RA_GN(TA, TW)                                                                                          \
+  add_group_rmsnorm_kernel<TA, TW><<<n_rows, threads, 0, stream>>>(resid, (const TA*)delta, (const TW*)weight, \
+                                                                   (TA*)out, rows, hidden, groups, eps, delta_scale)
+  if (act_dtype == RA_F32 && weight_dtype == RA_F32) RA_GN(float, float);
+  else if (act_dtype == RA_BF16 && weight_dtype == RA_BF16) RA_GN(bf16_t, bf16_t);
+  else if (act_dtype == RA_BF16 && weight_dtype == RA_F32) RA_GN(bf16_t, float);
+  else return ra_fail("add_group_rmsnorm: unsupported dtypes (activations %d, weight %d)", act_dtype, weight_dtype);
+#undef RA_GN
+  RA_LAUNCH_CHECK("add_group_rmsnorm");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
 // Fused per-head RMSNorm of q and k, rotation, and cache write.
 // qkv: [T, (Hq + 2 Hkv) * d]; q heads are normalised + rotated in place, k heads
 // are normalised + rotated and stored at the token's cache slot, v heads are
@@ -777,8 +833,14 @@ extern "C" int ra_qk_norm_rope_cache_sums(const float* parts, int n_ranges, cons
 // group == 0 gate is columns [0, I) and up [I, 2I); with group > 0 the two are
 // interleaved in runs of `group` columns, as the gated product kernel wants them.
 // ---------------------------------------------------------------------------
+// act 0: silu; act 1: the tanh form of gelu, 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
+__device__ __forceinline__ float gate_act(float g, int act) {
+  if (act == 1) return 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+  return g / (1.f + expf(-g));
+}
+
 template <typename TA>
-__global__ void silu_mul_kernel(const TA* __restrict__ gu, TA* __restrict__ out, int I, int group, size_t total) {
+__global__ void silu_mul_kernel(const TA* __restrict__ gu, TA* __restrict__ out, int I, int group, size_t total, int act) {
   size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   for (; idx < total; idx += stride) {
@@ -788,13 +850,13 @@ __global__ void silu_mul_kernel(const TA* __restrict__ gu, TA* __restrict__ out,
     const size_t ui = group > 0 ? gi + group : (size_t)I + i;
     const float g = to_f32(gu[t * 2 * I + gi]);
     const float u = to_f32(gu[t * 2 * I + ui]);
-    out[idx] = from_f32<TA>(g / (1.f + expf(-g)) * u);
+    out[idx] = from_f32<TA>(gate_act(g, act) * u);
   }
 }
 
 // eight outputs a thread, 16-byte loads and stores; I a multiple of 8, group 0 or a multiple of 8
 template <typename TA>
-__global__ void silu_mul_vec_kernel(const TA* __restrict__ gu, TA* __restrict__ out, int I, int group, size_t total8) {
+__global__ void silu_mul_vec_kernel(const TA* __restrict__ gu, TA* __restrict__ out, int I, int group, size_t total8, int act) {
   size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   const int I8 = I / 8;
@@ -808,8 +870,8 @@ __global__ void silu_mul_vec_kernel(const TA* __restrict__ gu, TA* __restrict__ 
     f32x4_raw u0 = Vec4<TA>::load(row + ui), u1 = Vec4<TA>::load(row + ui + 4);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      g0[e] = g0[e] / (1.f + expf(-g0[e])) * u0[e];
-      g1[e] = g1[e] / (1.f + expf(-g1[e])) * u1[e];
+      g0[e] = gate_act(g0[e], act) * u0[e];
+      g1[e] = gate_act(g1[e], act) * u1[e];
     }
     Vec4<TA>::store(out + idx * 8, g0);
     Vec4<TA>::store(out + idx * 8 + 4, g1);
@@ -818,7 +880,13 @@ __global__ void silu_mul_vec_kernel(const TA* __restrict__ gu, TA* __restrict__ 
 
 extern "C" int ra_silu_mul(const void* gate_up, void* out, int act_dtype, int n_tokens, int intermediate,
                            int group, hipStream_t stream) {
+  return ra_act_mul(gate_up, out, act_dtype, n_tokens, intermediate, group, 0, stream);
+}
+
+extern "C" int ra_act_mul(const void* gate_up, void* out, int act_dtype, int n_tokens, int intermediate,
+                          int group, int act, hipStream_t stream) {
   RA_CHECK(n_tokens > 0 && intermediate > 0, "silu_mul: empty input");
+  RA_CHECK(act == 0 || act == 1, "act_mul: unknown activation %d", act);
   RA_CHECK(group >= 0 && (group == 0 || intermediate % group == 0),
            "silu_mul: width %d is not a whole number of runs of %d", intermediate, group);
   const size_t total = (size_t)n_tokens * intermediate;
@@ -828,18 +896,18 @@ extern "C" int ra_silu_mul(const void* gate_up, void* out, int act_dtype, int n_
     size_t vb = (total8 + 255) / 256;
     if (vb > 65535 * 4) vb = 65535 * 4;
     if (act_dtype == RA_F32)
-      silu_mul_vec_kernel<float><<<(unsigned)vb, 256, 0, stream>>>((const float*)gate_up, (float*)out, intermediate, group, total8);
+      silu_mul_vec_kernel<float><<<(unsigned)vb, 256, 0, stream>>>((const float*)gate_up, (float*)out, intermediate, group, total8, act);
     else
-      silu_mul_vec_kernel<bf16_t><<<(unsigned)vb, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, intermediate, group, total8);
+      silu_mul_vec_kernel<bf16_t><<<(unsigned)vb, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, intermediate, group, total8, act);
     RA_LAUNCH_CHECK("silu_mul");
     return 0;
   }
   size_t blocks = (total + 255) / 256;
   if (blocks > 65535 * 4) blocks = 65535 * 4;
   if (act_dtype == RA_F32)
-    silu_mul_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>((const float*)gate_up, (float*)out, intermediate, group, total);
+    silu_mul_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>((const float*)gate_up, (float*)out, intermediate, group, total, act);
   else if (act_dtype == RA_BF16)
-    silu_mul_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, intermediate, group, total);
+    silu_mul_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, intermediate, group, total, act);
   else
     return ra_fail("silu_mul: unknown dtype tag %d", act_dtype);
   RA_LAUNCH_CHECK("silu_mul");

@@ -115,7 +115,7 @@ template <int MT>
 __global__ void __launch_bounds__(256)
 head_linear_mfma_kernel(const bf16_t* __restrict__ x, int ldx, int x_head, const bf16_t* __restrict__ W,
                         bf16_t* __restrict__ out, int ldo, int o_head, const bf16_t* __restrict__ gate, int ldg,
-                        int T, int N, int K) {
+                        int gate_per_head, int T, int N, int K) {
   const int lane = threadIdx.x & (RA_WAVE - 1);
   const int wave = threadIdx.x / RA_WAVE;
   const int r = lane & 15, g = lane >> 4;
@@ -157,7 +157,7 @@ head_linear_mfma_kernel(const bf16_t* __restrict__ x, int ldx, int x_head, const
       if (n >= N) continue;
       float v = acc[mt][i];
       if (gate) {
-        const float gv = to_f32(gate[(size_t)t * ldg + (size_t)h * N + n]);
+        const float gv = to_f32(gate[(size_t)t * ldg + (gate_per_head ? (size_t)h : (size_t)h * N + n)]);
         v *= 1.f / (1.f + expf(-gv));
       }
       out[(size_t)t * ldo + (size_t)h * o_head + n] = from_f32<bf16_t>(v);
@@ -169,7 +169,7 @@ head_linear_mfma_kernel(const bf16_t* __restrict__ x, int ldx, int x_head, const
 template <typename TA>
 __global__ void head_linear_kernel(const TA* __restrict__ x, int ldx, int x_head, const TA* __restrict__ W,
                                    TA* __restrict__ out, int ldo, int o_head, const TA* __restrict__ gate,
-                                   int ldg, int T, int N, int K) {
+                                   int ldg, int gate_per_head, int T, int N, int K) {
   extern __shared__ float xs[];          // [K][HL_TOKENS]
   const int h = blockIdx.x;
   const int t0 = blockIdx.y * HL_TOKENS;
@@ -202,7 +202,7 @@ __global__ void head_linear_kernel(const TA* __restrict__ x, int ldx, int x_head
       if (i < nt) {
         float v = acc[i];
         if (gate) {
-          const float g = to_f32(gate[(size_t)(t0 + i) * ldg + (size_t)h * N + n]);
+          const float g = to_f32(gate[(size_t)(t0 + i) * ldg + (gate_per_head ? (size_t)h : (size_t)h * N + n)]);
           v *= 1.f / (1.f + expf(-g));
         }
         out[(size_t)(t0 + i) * ldo + (size_t)h * o_head + n] = from_f32<TA>(v);
@@ -212,12 +212,12 @@ __global__ void head_linear_kernel(const TA* __restrict__ x, int ldx, int x_head
 }
 
 extern "C" int ra_head_linear(const void* x, int ldx, int x_head, const void* W, void* out, int ldo, int o_head,
-                              const void* gate, int ldg, int act_dtype, int n_tokens, int H, int N, int K,
-                              hipStream_t stream) {
+                              const void* gate, int ldg, int gate_per_head, int act_dtype, int n_tokens, int H,
+                              int N, int K, hipStream_t stream) {
   RA_CHECK(n_tokens > 0 && H > 0 && N > 0 && K > 0, "head_linear: %d tokens, %d heads, %d x %d", n_tokens, H, N, K);
   RA_CHECK(ldx >= (H - 1) * x_head + K && ldo >= (H - 1) * o_head + N && x_head >= 0 && o_head >= N,
            "head_linear: rows of %d / %d do not hold %d heads of %d / %d", ldx, ldo, H, K, N);
-  RA_CHECK(gate == nullptr || ldg >= H * N, "head_linear: gate rows of %d for %d heads of %d", ldg, H, N);
+  RA_CHECK(gate == nullptr || ldg >= (gate_per_head ? H : H * N), "head_linear: gate rows of %d for %d heads of %d", ldg, H, N);
   RA_CHECK(H <= 65535, "head_linear: %d heads in one launch", H);
   if (act_dtype == RA_BF16 && K % 8 == 0 && ldx % 8 == 0 && x_head % 8 == 0 && ((uintptr_t)x % 16) == 0 &&
       ((uintptr_t)W % 16) == 0) {
@@ -226,14 +226,14 @@ extern "C" int ra_head_linear(const void* x, int ldx, int x_head, const void* W,
       dim3 grid(col_groups, 1, H);
       head_linear_mfma_kernel<1><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, x_head, (const bf16_t*)W,
                                                            (bf16_t*)out, ldo, o_head, (const bf16_t*)gate, ldg,
-                                                           n_tokens, N, K);
+                                                           gate_per_head, n_tokens, N, K);
     } else {
       const int tiles = (n_tokens + 63) / 64;
       RA_CHECK(tiles <= 65535, "head_linear: %d tokens in one launch", n_tokens);
       dim3 grid(col_groups, tiles, H);
       head_linear_mfma_kernel<4><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, x_head, (const bf16_t*)W,
                                                            (bf16_t*)out, ldo, o_head, (const bf16_t*)gate, ldg,
-                                                           n_tokens, N, K);
+                                                           gate_per_head, n_tokens, N, K);
     }
     RA_LAUNCH_CHECK("head_linear");
     return 0;
@@ -249,11 +249,11 @@ extern "C" int ra_head_linear(const void* x, int ldx, int x_head, const void* W,
   if (act_dtype == RA_F32)
     head_linear_kernel<float><<<grid, threads, lds, stream>>>((const float*)x, ldx, x_head, (const float*)W,
                                                               (float*)out, ldo, o_head, (const float*)gate, ldg,
-                                                              n_tokens, N, K);
+                                                              gate_per_head, n_tokens, N, K);
   else if (act_dtype == RA_BF16)
     head_linear_kernel<bf16_t><<<grid, threads, lds, stream>>>((const bf16_t*)x, ldx, x_head, (const bf16_t*)W,
                                                                (bf16_t*)out, ldo, o_head, (const bf16_t*)gate, ldg,
-                                                               n_tokens, N, K);
+                                                               gate_per_head, n_tokens, N, K);
   else
     return ra_fail("head_linear: unknown dtype tag %d", act_dtype);
   RA_LAUNCH_CHECK("head_linear");

@@ -164,6 +164,148 @@ extern "C" int ra_moe_route_sigmoid(const float* logits, int ld, int experts, in
 }
 
 // ---------------------------------------------------------------------------
+// Softmax scores over all E outputs of the router with a correction that only the choice sees. One wave a
+// token: s = softmax(z) and the choice score c = s + correction go to LDS; with more than one group (equal runs
+// of neighbours) a group's score is its largest c, the `kept` best groups stay (ties: the lower group) and the
+// others' c become -inf; `top` rounds of a wave-wide maximum over c (ties: the lower index) choose; the weights
+// are the chosen s over their sum + norm_eps.
+// ---------------------------------------------------------------------------
+__global__ void moe_route_softmax_kernel(const float* __restrict__ logits, int ld, int E, int top, int groups,
+                                         int kept, const float* __restrict__ correction, float norm_eps,
+                                         int* __restrict__ ids, float* __restrict__ weights, int T) {
+  extern __shared__ float zs[];          // [MOE_TOPK_WAVES][2 E + groups]
+  const int lane = threadIdx.x & (RA_WAVE - 1);
+  const int wave = threadIdx.x / RA_WAVE;
+  const int t = blockIdx.x * MOE_TOPK_WAVES + wave;
+  if (t >= T) return;                    // whole waves leave; no workgroup barrier below
+  float* s = zs + (size_t)wave * (2 * E + groups);
+  float* c = s + E;
+  float* gs = c + E;
+  float m = -INFINITY;
+  for (int e = lane; e < E; e += RA_WAVE) m = fmaxf(m, logits[(size_t)t * ld + e]);
+  m = wave_max(m);
+  float sum = 0.f;
+  for (int e = lane; e < E; e += RA_WAVE) {
+    const float p = expf(logits[(size_t)t * ld + e] - m);
+    s[e] = p;
+    sum += p;
+  }
+  sum = wave_sum(sum);
+  for (int e = lane; e < E; e += RA_WAVE) {      // a lane reads back only what it wrote itself
+    const float p = s[e] / sum;
+    s[e] = p;
+    c[e] = p + (correction ? correction[e] : 0.f);
+  }
+  __builtin_amdgcn_wave_barrier();
+  if (groups > 1) {
+    const int size = E / groups;
+    for (int g = lane; g < groups; g += RA_WAVE) {
+      float best = -INFINITY;
+      for (int i = 0; i < size; ++i) best = fmaxf(best, c[g * size + i]);
+      gs[g] = best;
+    }
+    __builtin_amdgcn_wave_barrier();
+    for (int j = 0; j < kept; ++j) {
+      float best = -INFINITY;
+      int at = 0x7fffffff;
+      for (int g = lane; g < groups; g += RA_WAVE) {
+        const float v = gs[g];
+        if (v != INFINITY && (at == 0x7fffffff || v > best)) { best = v; at = g; }
+      }
+#pragma unroll
+      for (int mm = RA_WAVE / 2; mm > 0; mm >>= 1) {
+        const float ob = __shfl_xor(best, mm, RA_WAVE);
+        const int oa = __shfl_xor(at, mm, RA_WAVE);
+        if (oa != 0x7fffffff && (at == 0x7fffffff || ob > best || (ob == best && oa < at))) { best = ob; at = oa; }
+      }
+      if (at < groups && (at & (RA_WAVE - 1)) == lane) gs[at] = INFINITY;
+      __builtin_amdgcn_wave_barrier();
+    }
+    for (int e = lane; e < E; e += RA_WAVE)
+      if (gs[e / size] != INFINITY) c[e] = -INFINITY;
+    __builtin_amdgcn_wave_barrier();
+  }
+  float mine = 0.f, total = 0.f;
+  int mine_id = 0;
+  for (int j = 0; j < top; ++j) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+    for (int e = lane; e < E; e += RA_WAVE) {
+      const float v = c[e];
+      if (at == 0x7fffffff || v > best) { best = v; at = e; }
+    }
+#pragma unroll
+    for (int mm = RA_WAVE / 2; mm > 0; mm >>= 1) {
+      const float ob = __shfl_xor(best, mm, RA_WAVE);
+      const int oa = __shfl_xor(at, mm, RA_WAVE);
+      if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+    }
+    const float p = s[at];                 // every lane reads the winner's score: written before the barrier above
+    total += p;
+    if (lane == j) { mine = p; mine_id = at; }
+    if ((at & (RA_WAVE - 1)) == lane) c[at] = -INFINITY;
+  }
+  if (lane < top) {
+    weights[(size_t)t * top + lane] = mine / (total + norm_eps);
+    ids[(size_t)t * top + lane] = mine_id;
+  }
+}
+
+extern "C" int ra_moe_route_softmax(const float* logits, int ld, int experts, int top, int groups, int kept,
+                                    const float* correction, float norm_eps, int* ids, float* weights, int n_tokens,
+                                    hipStream_t stream) {
+  RA_CHECK(n_tokens > 0 && experts > 0, "moe_route_softmax: %d tokens, %d experts", n_tokens, experts);
+  RA_CHECK(groups >= 1 && experts % groups == 0 && kept >= 1 && kept <= groups,
+           "moe_route_softmax: %d experts in %d groups, %d kept", experts, groups, kept);
+  RA_CHECK(top > 0 && top <= RA_WAVE && top <= kept * (experts / groups),
+           "moe_route_softmax: %d of %d experts that can be chosen (at most 64)", top, kept * (experts / groups));
+  RA_CHECK(ld >= experts, "moe_route_softmax: rows of %d for %d experts", ld, experts);
+  const size_t lds = (size_t)MOE_TOPK_WAVES * (2 * experts + groups) * sizeof(float);
+  RA_CHECK(lds <= 64 * 1024, "moe_route_softmax: %d experts", experts);
+  const int blocks = (n_tokens + MOE_TOPK_WAVES - 1) / MOE_TOPK_WAVES;
+  moe_route_softmax_kernel<<<blocks, MOE_TOPK_WAVES * RA_WAVE, lds, stream>>>(logits, ld, experts, top, groups, kept,
+                                                                              correction, norm_eps, ids, weights,
+                                                                              n_tokens);
+  RA_LAUNCH_CHECK("moe_route_softmax");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Identity experts: a chosen id of E or more names no matrices; its output is the token's input row. One
+// workgroup a token: y[t, :] += (sum of the weights of such choices) * x[t, :], the sum and product in float.
+// ---------------------------------------------------------------------------
+template <typename TA>
+__global__ void moe_identity_add_kernel(TA* __restrict__ y, int ldy, const TA* __restrict__ x, int ldx,
+                                        const int* __restrict__ ids, const float* __restrict__ weights, int top, int E,
+                                        int width) {
+  const size_t t = blockIdx.x;
+  float coef = 0.f;
+  for (int j = 0; j < top; ++j)
+    if (ids[t * top + j] >= E) coef += weights[t * top + j];
+  if (coef == 0.f) return;
+  for (int e = threadIdx.x; e < width; e += blockDim.x)
+    y[t * ldy + e] = from_f32<TA>(to_f32(y[t * ldy + e]) + coef * to_f32(x[t * ldx + e]));
+}
+
+extern "C" int ra_moe_identity_add(void* y, int ldy, const void* x, int ldx, int act_dtype, const int* ids,
+                                   const float* weights, int top, int experts, int n_tokens, int width,
+                                   hipStream_t stream) {
+  RA_CHECK(n_tokens > 0 && width > 0 && top > 0 && ldy >= width && ldx >= width,
+           "moe_identity_add: %d tokens, width %d, %d choices", n_tokens, width, top);
+  const int threads = width >= 1024 ? 256 : width >= 256 ? 128 : 64;
+  if (act_dtype == RA_F32)
+    moe_identity_add_kernel<float><<<n_tokens, threads, 0, stream>>>((float*)y, ldy, (const float*)x, ldx, ids, weights,
+                                                                     top, experts, width);
+  else if (act_dtype == RA_BF16)
+    moe_identity_add_kernel<bf16_t><<<n_tokens, threads, 0, stream>>>((bf16_t*)y, ldy, (const bf16_t*)x, ldx, ids,
+                                                                      weights, top, experts, width);
+  else
+    return ra_fail("moe_identity_add: unknown dtype tag %d", act_dtype);
+  RA_LAUNCH_CHECK("moe_identity_add");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
 // Gated experts side by side: gu[t, e * 2 ff + j] is expert e's gate projection of token t and
 // gu[t, e * 2 ff + ff + j] its up projection; behind the experts a shared expert's [gate | up] of `shared` each.
 // act[t, e * ff + j] = p(t, e) * silu(gate) * up for the chosen experts and 0 for the others;
@@ -172,12 +314,16 @@ extern "C" int ra_moe_route_sigmoid(const float* logits, int ld, int experts, in
 template <typename TA>
 __global__ void moe_silu_gate_scale_kernel(const TA* __restrict__ gu, TA* __restrict__ act,
                                            const int* __restrict__ ids, const float* __restrict__ weights, int top,
-                                           int E, int ff, int shared) {
+                                           int E, int ff, int shared, const float* __restrict__ shared_logit,
+                                           int ld_logit) {
   extern __shared__ float gate[];        // [E]
   const int t = blockIdx.y;
   for (int e = threadIdx.x; e < E; e += blockDim.x) gate[e] = 0.f;
   __syncthreads();
-  for (int j = threadIdx.x; j < top; j += blockDim.x) gate[ids[(size_t)t * top + j]] = weights[(size_t)t * top + j];
+  for (int j = threadIdx.x; j < top; j += blockDim.x) {
+    const int id = ids[(size_t)t * top + j];
+    if (id < E) gate[id] = weights[(size_t)t * top + j];     // an id past the experts names no matrices (an identity expert)
+  }
   __syncthreads();
   const int n = E * ff + shared;
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -195,7 +341,7 @@ __global__ void moe_silu_gate_scale_kernel(const TA* __restrict__ gu, TA* __rest
     u = to_f32(row[(size_t)e * 2 * ff + ff + j]);
   } else {
     const int j = i - E * ff;
-    p = 1.f;
+    p = shared_logit ? 1.f / (1.f + expf(-shared_logit[(size_t)t * ld_logit])) : 1.f;
     g = to_f32(row[(size_t)E * 2 * ff + j]);
     u = to_f32(row[(size_t)E * 2 * ff + shared + j]);
   }
@@ -204,7 +350,15 @@ __global__ void moe_silu_gate_scale_kernel(const TA* __restrict__ gu, TA* __rest
 
 extern "C" int ra_moe_silu_gate_scale(const void* gu, void* act, int act_dtype, const int* ids, const float* weights,
                                       int top, int experts, int ff, int shared, int n_tokens, hipStream_t stream) {
-  RA_CHECK(n_tokens > 0 && experts > 0 && ff > 0 && top > 0 && top <= experts && shared >= 0,
+  return ra_moe_silu_gate_scale_shared(gu, act, act_dtype, ids, weights, top, experts, ff, shared, nullptr, 0, n_tokens,
+                                       stream);
+}
+
+extern "C" int ra_moe_silu_gate_scale_shared(const void* gu, void* act, int act_dtype, const int* ids,
+                                             const float* weights, int top, int experts, int ff, int shared,
+                                             const float* shared_logit, int ld_logit, int n_tokens,
+                                             hipStream_t stream) {
+  RA_CHECK(n_tokens > 0 && experts > 0 && ff > 0 && top > 0 && shared >= 0,
            "moe_silu_gate_scale: %d tokens, %d of %d experts of %d, shared %d", n_tokens, top, experts, ff, shared);
   RA_CHECK(n_tokens <= 65535, "moe_silu_gate_scale: %d tokens in one launch (max 65535)", n_tokens);
   const size_t lds = (size_t)experts * sizeof(float);
@@ -213,10 +367,10 @@ extern "C" int ra_moe_silu_gate_scale(const void* gu, void* act, int act_dtype, 
   dim3 grid((n + 255) / 256, n_tokens);
   if (act_dtype == RA_F32)
     moe_silu_gate_scale_kernel<float><<<grid, 256, lds, stream>>>((const float*)gu, (float*)act, ids, weights, top,
-                                                                   experts, ff, shared);
+                                                                   experts, ff, shared, shared_logit, ld_logit);
   else if (act_dtype == RA_BF16)
     moe_silu_gate_scale_kernel<bf16_t><<<grid, 256, lds, stream>>>((const bf16_t*)gu, (bf16_t*)act, ids, weights, top,
-                                                                    experts, ff, shared);
+                                                                    experts, ff, shared, shared_logit, ld_logit);
   else
     return ra_fail("moe_silu_gate_scale: unknown dtype tag %d", act_dtype);
   RA_LAUNCH_CHECK("moe_silu_gate_scale");

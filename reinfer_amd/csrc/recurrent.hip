@@ -19,7 +19,8 @@ struct ScanGeom {
   int wave_floats;             // floats of state a wave
 };
 
-// kind 0: matrix memory (S, the normaliser n once a wave, the running maximum m); kind 1: delta rule (S)
+// kind 0: matrix memory (S, the normaliser n once a wave, the running maximum m); kind 1: delta rule (S);
+// kind 2: wkv (S)
 bool scan_geom(int kind, int dk, int dv, ScanGeom* g) {
   if (dk <= 0 || dv <= 0 || dk > 512) return false;
   // at most 8 elements a lane: the per-token chain of multiply-adds stays short, and a head has enough waves to
@@ -75,6 +76,8 @@ __device__ __forceinline__ float logsigmoid_f(float x) { return -softplus_f(-x);
 #define SCAN_CHUNK_MAX 16
 #define SCAN_LDS_FLOATS 6144   // of one of the two buffers
 
+enum { SCAN_DELTA = 0, SCAN_MEMORY = 1, SCAN_WKV = 2 };
+
 struct ScanArgs {
   const void* q; const void* k; const void* v;     // column 0 of each in row 0; rows ld elements apart
   int ld;
@@ -85,13 +88,18 @@ struct ScanArgs {
   int H, dk, dv, waves_per_head, wave_floats, chunk;
   float q_scale, denom_eps;
   float* out;
+  // wkv: the decays' pre-activations, float [T, H dk] with rows ldw apart, their bias w0 [H dk] and the bonus u [H dk]
+  const float* w; int ldw; const float* w0; const float* u;
 };
 
-template <typename TA, int R, int NPL, bool MEMORY>
+template <typename TA, int R, int NPL, int MODE>
 __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
+  constexpr bool MEMORY = MODE == SCAN_MEMORY, WKV = MODE == SCAN_WKV;
   constexpr int CPW = RA_WAVE / R;
   constexpr int PITCH = NPL + 4;                     // floats of a lane's run of k (or q) in LDS, padded
-  constexpr int NG = MEMORY ? 3 : 2;                 // gate values a token
+  constexpr int NG = MEMORY ? 3 : WKV ? 0 : 2;       // gate values a token
+  constexpr int NGD = NG ? NG : 1;
+  constexpr int NV = WKV ? 3 : 2;                    // vectors over the key size a token: k, q and, for wkv, the decay
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int seq = blockIdx.x, head = blockIdx.y;
   const int tid = threadIdx.x, nthreads = blockDim.x;
@@ -113,15 +121,18 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
     return;
   }
   if (first >= last) return;
-  // LDS: two buffers of [CT][2][R][PITCH] k and q, [CT][cols] v, [CT][NG] gates
-  const int kq_floats = CT * 2 * R * PITCH, v_floats = CT * cols;
+  // LDS: two buffers of [CT][NV][R][PITCH] k, q (and the decay), [CT][cols] v, [CT][NG] gates
+  const int kq_floats = CT * NV * R * PITCH, v_floats = CT * cols;
   const int buf_floats = kq_floats + v_floats + CT * NG;
   const int qh = head / (H / p.q_heads);
   const TA* qg = (const TA*)p.q + (size_t)qh * dk;
   const TA* kg = (const TA*)p.k + (size_t)qh * dk;
   const TA* vg = (const TA*)p.v + (size_t)head * dv + (size_t)blockIdx.z * cols;
   const int v_left = dv - blockIdx.z * cols;         // columns of this workgroup that exist
-  float fk[SCAN_KQ_REGS], fq[SCAN_KQ_REGS], fv[SCAN_V_REGS], fg = 0.f;
+  float fk[SCAN_KQ_REGS], fq[SCAN_KQ_REGS], fw[WKV ? SCAN_KQ_REGS : 1], fv[SCAN_V_REGS], fg = 0.f;
+  const float* wg = WKV ? p.w + (size_t)head * dk : nullptr;
+  const float* w0 = WKV ? p.w0 + (size_t)head * dk : nullptr;
+  int kq_w[WKV ? SCAN_KQ_REGS : 1];                  // the decay's place: rows of its own pitch, the bias by element
   // what this thread fetches for a chunk is the same for every chunk: token (of the chunk), offset behind the
   // chunk's first row, and place in LDS are worked out once
   int kq_t[SCAN_KQ_REGS], kq_g[SCAN_KQ_REGS], kq_l[SCAN_KQ_REGS];
@@ -133,7 +144,8 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
     kq_t[j] = t < CT ? t : SCAN_CHUNK_MAX;           // past the chunk: never fetched, never stored
     kq_e[j] = e < dk;
     kq_g[j] = t * p.ld + e;
-    kq_l[j] = t * 2 * R * PITCH + (e / NPL) * PITCH + (e % NPL);
+    kq_l[j] = t * NV * R * PITCH + (e / NPL) * PITCH + (e % NPL);
+    if (WKV) kq_w[j] = e;
   }
   int v_t[SCAN_V_REGS], v_g[SCAN_V_REGS];
 #pragma unroll
@@ -143,7 +155,7 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
     v_t[j] = (t < CT && cc < v_left) ? t : SCAN_CHUNK_MAX;
     v_g[j] = t * p.ld + cc;
   }
-  const int g_t = tid < NG * CT ? tid / NG : SCAN_CHUNK_MAX;
+  const int g_t = tid < NG * CT ? tid / NGD : SCAN_CHUNK_MAX;
   const int g_g = g_t * NG * H + (tid - g_t * NG) * H + head;
   auto fetch = [&](int t0) {                         // chunk starting at token t0 -> registers
     const int n = min(CT, last - t0);
@@ -155,10 +167,15 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
         fk[j] = to_f32(kg[row0 + kq_g[j]]);
         fq[j] = to_f32(qg[row0 + kq_g[j]]) * p.q_scale;
       }
+      if (WKV) {                                     // the decay exp(-exp(z + w0)), float from its pre-activation on
+        fw[j] = 0.f;
+        if (kq_t[j] < n && kq_e[j])
+          fw[j] = expf(-expf(wg[(size_t)(t0 + kq_t[j]) * p.ldw + kq_w[j]] + w0[kq_w[j]]));
+      }
     }
 #pragma unroll
     for (int j = 0; j < SCAN_V_REGS; ++j) fv[j] = v_t[j] < n ? to_f32(vg[row0 + v_g[j]]) : 0.f;
-    fg = g_t < n ? p.gates[(size_t)t0 * NG * H + g_g] : 0.f;
+    fg = (NG && g_t < n) ? p.gates[(size_t)t0 * NG * H + g_g] : 0.f;
   };
   auto stage = [&](float* buf) {                     // registers -> LDS
 #pragma unroll
@@ -166,6 +183,7 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
       if (kq_t[j] < SCAN_CHUNK_MAX) {
         buf[kq_l[j]] = fk[j];
         buf[kq_l[j] + R * PITCH] = fq[j];
+        if (WKV) buf[kq_l[j] + 2 * R * PITCH] = fw[j];
       }
     }
 #pragma unroll
@@ -173,15 +191,16 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
       const int idx = tid + j * nthreads;
       if (idx < v_floats) buf[kq_floats + idx] = fv[j];
     }
-    if (tid < NG * CT) buf[kq_floats + v_floats + tid] = fg;
+    if (NG && tid < NG * CT) buf[kq_floats + v_floats + tid] = fg;
   };
   float* st = p.state + (size_t)slot * p.slot_stride + (size_t)(head * p.waves_per_head + (active ? w : 0)) * p.wave_floats;
   const bool zero = p.fresh[seq] != 0;
-  float S[NPL], nrm[NPL];
+  float S[NPL], nrm[NPL], bonus[NPL];
 #pragma unroll
   for (int i = 0; i < NPL; ++i) {
     S[i] = (zero || !active) ? 0.f : st[i * RA_WAVE + lane];
     nrm[i] = 0.f;
+    bonus[i] = (WKV && r * NPL + i < dk) ? p.u[(size_t)head * dk + r * NPL + i] : 0.f;
     if (MEMORY && !zero && active) nrm[i] = st[NPL * RA_WAVE + i * R + r];
   }
   fetch(first);
@@ -195,15 +214,19 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
     const int n = min(CT, last - t0);
     if (active) {
       const int vcol = (tid / RA_WAVE) * CPW + c;
-      struct Operands { float k[NPL], q[NPL], v, g0, g1, g2; };
+      struct Operands { float k[NPL], q[NPL], w[WKV ? NPL : 1], v, g0, g1, g2; };
       auto read = [&](int tt, Operands& x) {         // a token's operands out of LDS
-        const float* kp = buf + (size_t)tt * 2 * R * PITCH + r * PITCH;
+        const float* kp = buf + (size_t)tt * NV * R * PITCH + r * PITCH;
         const float* qp = kp + R * PITCH;
 #pragma unroll
         for (int i = 0; i < NPL; ++i) { x.k[i] = kp[i]; x.q[i] = qp[i]; }
+        if (WKV) {
+#pragma unroll
+          for (int i = 0; i < NPL; ++i) x.w[i] = qp[R * PITCH + i];
+        }
         x.v = buf[kq_floats + tt * cols + vcol];
-        x.g0 = buf[kq_floats + v_floats + NG * tt];
-        x.g1 = buf[kq_floats + v_floats + NG * tt + 1];
+        x.g0 = NG ? buf[kq_floats + v_floats + NG * tt] : 0.f;
+        x.g1 = NG ? buf[kq_floats + v_floats + NG * tt + 1] : 0.f;
         x.g2 = MEMORY ? buf[kq_floats + v_floats + NG * tt + 2] : 0.f;
       };
       auto step = [&](int tt, const Operands& x) {   // one token: the state moves on, the read-out is stored
@@ -222,6 +245,16 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
           const float s1 = group_sum<R>(ps[0] + ps[1]);
           const float s2 = group_sum<R>(pn[0] + pn[1]);
           o = __fdividef(s1, fmaxf(fabsf(s2), x.g2) + p.denom_eps);      // a reciprocal and a product: within an ulp or two
+        } else if (WKV) {
+          // o = (S + diag(u) k v^T)^T q with the bonus for this token alone; then S <- diag(w) S + k v^T
+          float po[2] = {0.f, 0.f};
+#pragma unroll
+          for (int i = 0; i < NPL; ++i) {
+            const float kv = x.k[i] * x.v;
+            po[i & 1] += x.q[i] * (S[i] + bonus[i] * kv);
+            S[i] = x.w[i] * S[i] + kv;
+          }
+          o = group_sum<R>(po[0] + po[1]);
         } else {
           float pa[2] = {0.f, 0.f}, pb[2] = {0.f, 0.f}, pkq[2] = {0.f, 0.f};
 #pragma unroll
@@ -521,13 +554,13 @@ struct ScanLaunch {
   int threads, chunk;
   size_t lds;
 };
-ScanLaunch scan_launch(const ScanGeom& g, int n_seqs, int heads, int max_q_len) {
+ScanLaunch scan_launch(const ScanGeom& g, int n_seqs, int heads, int max_q_len, int vectors = 2) {
   const int wpb = g.waves < 4 ? g.waves : 4;           // waves a workgroup
   ScanLaunch L;
   L.threads = wpb * RA_WAVE;
   L.grid = dim3(n_seqs, heads, (g.waves + wpb - 1) / wpb);
   const int cols = wpb * g.CPW;
-  const int per_token = 2 * g.R * (g.NPL + 4) + cols + 3;      // k and q runs, the columns of v, up to 3 gate numbers
+  const int per_token = vectors * g.R * (g.NPL + 4) + cols + 3;      // k and q (and decay) runs, the columns of v, up to 3 gate numbers
   int ct = SCAN_CHUNK_MAX;
   if (ct > SCAN_KQ_REGS * L.threads / (g.R * g.NPL)) ct = SCAN_KQ_REGS * L.threads / (g.R * g.NPL);
   if (max_q_len > 0 && ct > max_q_len) ct = max_q_len;      // a step of single tokens stages one token
@@ -540,7 +573,7 @@ ScanLaunch scan_launch(const ScanGeom& g, int n_seqs, int heads, int max_q_len) 
   return L;
 }
 
-template <typename TA, bool MEMORY>
+template <typename TA, int MEMORY>
 int scan_dispatch(const ScanGeom& g, const ScanLaunch& L, const ScanArgs& a, hipStream_t stream) {
 #define RA_SCAN(R, NPL) scan_kernel<TA, R, NPL, MEMORY><<<L.grid, L.threads, L.lds, stream>>>(a)
 #define RA_SCAN_N(R)                               \
@@ -589,8 +622,8 @@ extern "C" int ra_matrix_memory_scan(const void* proj, int act_dtype, int ld, in
   a.cu_tokens = cu_tokens; a.state_slots = state_slots; a.fresh = fresh;
   a.H = heads; a.dk = key_dim; a.dv = value_dim; a.waves_per_head = g.waves; a.wave_floats = g.wave_floats;
   a.chunk = L.chunk; a.q_scale = q_scale; a.denom_eps = denom_eps; a.out = out;
-  if (act_dtype == RA_F32) scan_dispatch<float, true>(g, L, a, stream);
-  else scan_dispatch<bf16_t, true>(g, L, a, stream);
+  if (act_dtype == RA_F32) scan_dispatch<float, SCAN_MEMORY>(g, L, a, stream);
+  else scan_dispatch<bf16_t, SCAN_MEMORY>(g, L, a, stream);
   RA_LAUNCH_CHECK("matrix_memory_scan");
   return 0;
 }
@@ -651,8 +684,37 @@ extern "C" int ra_delta_rule_scan(const float* qkv, int ld, float* gates, const 
   a.cu_tokens = cu_tokens; a.state_slots = state_slots; a.fresh = fresh;
   a.H = heads; a.dk = key_dim; a.dv = value_dim; a.waves_per_head = g.waves; a.wave_floats = g.wave_floats;
   a.chunk = L.chunk; a.q_scale = 1.f; a.denom_eps = 0.f; a.out = out;
-  scan_dispatch<float, false>(g, L, a, stream);
+  scan_dispatch<float, SCAN_DELTA>(g, L, a, stream);
   RA_LAUNCH_CHECK("delta_rule_scan");
+  return 0;
+}
+
+extern "C" int ra_wkv_scan(const void* proj, int act_dtype, int ld, int r_off, int k_off, int v_off, const float* decay,
+                           int ldw, const float* w0, const float* u, float* state, long slot_stride,
+                           const int* cu_tokens, const int* state_slots, const int* fresh, int n_seqs, int n_tokens,
+                           int max_q_len, int heads, int dim, float* out, hipStream_t stream) {
+  RA_CHECK(n_seqs > 0 && n_tokens > 0 && heads > 0, "wkv_scan: %d requests, %d tokens, %d heads", n_seqs, n_tokens, heads);
+  ScanGeom g;
+  RA_CHECK(scan_geom(2, dim, dim, &g), "wkv_scan: heads of %d x %d (keys up to 512)", dim, dim);
+  RA_CHECK(slot_stride >= (long)heads * g.waves * g.wave_floats, "wkv_scan: a state slot of %ld floats, need %ld",
+           slot_stride, (long)heads * g.waves * g.wave_floats);
+  RA_CHECK(heads <= 65535, "wkv_scan: %d heads in one launch", heads);
+  RA_CHECK(ldw >= heads * dim, "wkv_scan: decay rows of %d for %d heads of %d", ldw, heads, dim);
+  RA_CHECK(act_dtype == RA_F32 || act_dtype == RA_BF16, "wkv_scan: unknown dtype tag %d", act_dtype);
+  const ScanLaunch L = scan_launch(g, n_seqs, heads, max_q_len, 3);
+  const size_t es = act_dtype == RA_F32 ? 4 : 2;
+  ScanArgs a = {};
+  a.q = (const char*)proj + (size_t)r_off * es;
+  a.k = (const char*)proj + (size_t)k_off * es;
+  a.v = (const char*)proj + (size_t)v_off * es;
+  a.ld = ld; a.q_heads = heads; a.gates = nullptr; a.state = state; a.slot_stride = slot_stride;
+  a.cu_tokens = cu_tokens; a.state_slots = state_slots; a.fresh = fresh;
+  a.H = heads; a.dk = dim; a.dv = dim; a.waves_per_head = g.waves; a.wave_floats = g.wave_floats;
+  a.chunk = L.chunk; a.q_scale = 1.f; a.denom_eps = 0.f; a.out = out;
+  a.w = decay; a.ldw = ldw; a.w0 = w0; a.u = u;
+  if (act_dtype == RA_F32) scan_dispatch<float, SCAN_WKV>(g, L, a, stream);
+  else scan_dispatch<bf16_t, SCAN_WKV>(g, L, a, stream);
+  RA_LAUNCH_CHECK("wkv_scan");
   return 0;
 }
 

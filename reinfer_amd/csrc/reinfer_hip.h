@@ -5,7 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define RA_ABI_VERSION 20
+#define RA_ABI_VERSION 21
 
 #ifdef __cplusplus
 extern "C" {
@@ -20,6 +20,11 @@ int ra_embed(const void* table, int table_dtype, const int* ids, float* out, int
 int ra_add_rmsnorm(float* resid, const void* delta, const void* weight, int weight_dtype, void* out,
                    int act_dtype, const int* rows, int n_rows, int hidden, float eps, float delta_scale,
                    hipStream_t stream);
+
+// The same norm in `groups` equal consecutive parts of the row, each over its own root mean square.
+int ra_add_group_rmsnorm(float* resid, const void* delta, const void* weight, int weight_dtype, void* out,
+                         int act_dtype, const int* rows, int n_rows, int hidden, int groups, float eps,
+                         float delta_scale, hipStream_t stream);
 
 int ra_qk_norm_rope_cache(void* qkv, int act_dtype, const void* q_weight, const void* k_weight,
                           int weight_dtype, float eps, const int* positions, const float* inv_freq,
@@ -38,6 +43,9 @@ int ra_qk_norm_rope_cache_sums(const float* parts, int n_ranges, const float* in
 // up interleaved in runs of `group` columns (gate run, then the up run of the same features)
 int ra_silu_mul(const void* gate_up, void* out, int act_dtype, int n_tokens, int intermediate,
                 int group, hipStream_t stream);
+// out = act(gate) * up; act 0: silu, act 1: the tanh form of gelu
+int ra_act_mul(const void* gate_up, void* out, int act_dtype, int n_tokens, int intermediate, int group, int act,
+               hipStream_t stream);
 
 int ra_attention_plain(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
                        const void* vcache, int act_dtype, const int* block_tables, int max_blocks,
@@ -189,9 +197,11 @@ int ra_latent_prep(const void* proj, int act_dtype, int ld, int q_off, int dkv_o
                    int weight_dtype, float eps, const int* positions, const float* inv_freq, int rot_dims, int R,
                    int rank, int H, int D, void* q_lat, int Dp, const int* slots, void* kcache, void* vcache,
                    int block_size, int n_tokens, hipStream_t stream);
-// out[t, h * o_head + n] = sum_k x[t, h * x_head + k] * W[h, k, n] (* sigmoid(gate[t, h * N + n]) if gate)
+// out[t, h * o_head + n] = sum_k x[t, h * x_head + k] * W[h, k, n] (* sigmoid(gate[t, h * N + n]) if gate, or
+// * sigmoid(gate[t, h]) with gate_per_head: one number a head)
 int ra_head_linear(const void* x, int ldx, int x_head, const void* W, void* out, int ldo, int o_head,
-                   const void* gate, int ldg, int act_dtype, int n_tokens, int H, int N, int K, hipStream_t stream);
+                   const void* gate, int ldg, int gate_per_head, int act_dtype, int n_tokens, int H, int N, int K,
+                   hipStream_t stream);
 
 // ---- mixture of experts (moe.hip) ----
 // the `top` (<= 64) largest of each row of float logits [n_tokens, experts] (row stride ld) in falling order into
@@ -219,6 +229,22 @@ int ra_moe_route_sigmoid(const float* logits, int ld, int experts, int top, int 
 // act [n_tokens, experts ff + shared] = weight * silu(gate) * up (0 for experts not chosen, weight 1 for the shared one)
 int ra_moe_silu_gate_scale(const void* gu, void* act, int act_dtype, const int* ids, const float* weights, int top,
                            int experts, int ff, int shared, int n_tokens, hipStream_t stream);
+
+// The same with the shared expert's weight sigmoid(shared_logit[t * ld_logit]) (float; null: weight 1); chosen ids
+// of `experts` or more name no matrices and are skipped
+int ra_moe_silu_gate_scale_shared(const void* gu, void* act, int act_dtype, const int* ids, const float* weights,
+                                  int top, int experts, int ff, int shared, const float* shared_logit, int ld_logit,
+                                  int n_tokens, hipStream_t stream);
+// softmax scores over all `experts` router outputs; the choice is by score + correction (float [experts], may be
+// null) inside the `kept` best of `groups` groups of neighbours (a group's score: its largest choice score); the
+// weights are the chosen scores over their sum + norm_eps
+int ra_moe_route_softmax(const float* logits, int ld, int experts, int top, int groups, int kept,
+                         const float* correction, float norm_eps, int* ids, float* weights, int n_tokens,
+                         hipStream_t stream);
+// y[t, :] += (sum of weights[t, j] with ids[t, j] >= experts) * x[t, :]: chosen ids past the experts stand for the
+// identity
+int ra_moe_identity_add(void* y, int ldy, const void* x, int ldx, int act_dtype, const int* ids, const float* weights,
+                        int top, int experts, int n_tokens, int width, hipStream_t stream);
 
 // C += acc_scale * (A . W^T) through the weight-streaming kernels (bfloat16 operands, float C; the limits of
 // ra_gemm_skinny / ra_gemm_wide with the accumulating epilogue)
@@ -250,11 +276,35 @@ int ra_delta_rule_scan(const float* qkv, int ld, float* gates, const float* a_lo
                        long slot_stride, const int* cu_tokens, const int* state_slots, const int* fresh, int n_seqs,
                        int n_tokens, int max_q_len, int heads, int key_heads, int key_dim, int value_dim, float* out,
                        hipStream_t stream);
+// kind 2 of ra_scan_state_floats. proj rows hold r, k and v (heads x dim each) at the given column offsets; decay
+// float [n_tokens, >= heads dim] holds the decays' pre-activations z, the decay being exp(-exp(z + w0)); u float
+// [heads dim] is the bonus of the current token: o = (S + diag(u) k v^T)^T r, then S <- diag(decay) S + k v^T
+int ra_wkv_scan(const void* proj, int act_dtype, int ld, int r_off, int k_off, int v_off, const float* decay, int ldw,
+                const float* w0, const float* u, float* state, long slot_stride, const int* cu_tokens,
+                const int* state_slots, const int* fresh, int n_seqs, int n_tokens, int max_q_len, int heads, int dim,
+                float* out, hipStream_t stream);
 int ra_head_norm_gate(const float* read, const float* weight, int per_head_weight, const void* gate, int ldg,
                       int act_dtype, int silu, float eps, int n_tokens, int heads, int value_dim, void* out,
                       hipStream_t stream);
 int ra_normed_mean(const void* const* xs, const float* const* ws, int n, int act_dtype, float eps, int n_tokens,
                    int hidden, void* out, float* resid, float scale, hipStream_t stream);
+
+// ---- around a mixer that reads the token before (shift.hip) ----
+// out[t, j width + e] = h[t, e] + (prev(t)[e] - h[t, e]) * mu[j, e] for j < n_mix; prev(t) is row t - 1 inside a
+// portion and, for a portion's first row, the row kept at keep_off floats in the request's state slot (zeros at a
+// request's start; state slot -1 reads zeros and keeps nothing). The slot then takes the portion's last row.
+// single_tokens != 0 promises that every request of the step brings one token (one launch instead of two).
+int ra_token_shift(const void* h, int ldh, const void* mu, int mu_dtype, int n_mix, float* state, long slot_stride,
+                   long keep_off, const int* seq_of_token, const int* cu_tokens, const int* state_slots,
+                   const int* fresh, void* out, int ldo, int act_dtype, int n_seqs, int n_tokens, int width,
+                   int single_tokens, hipStream_t stream);
+// resid[t, e] += sigmoid(gates[t, e]) * a[t, e] + sigmoid(gates[t, width + e]) * b[t, e]; b may be null
+int ra_gated_stream_add(float* resid, const void* gates, int ldg, int gate_dtype, const void* a, int a_dtype,
+                        const void* b, int b_dtype, int n_tokens, int width, hipStream_t stream);
+// out[r, :] = x[r, :] / sqrt(mean(x[r, :]^2) + eps) * weight over rows of activations ldx / ldo apart
+int ra_rows_rmsnorm(const void* x, int ldx, const void* weight, int weight_dtype, void* out, int ldo, int act_dtype,
+                    int n_rows, int width, float eps, hipStream_t stream);
+int ra_tanh_rows(void* x, int act_dtype, long n, hipStream_t stream);
 
 #ifdef __cplusplus
 }

@@ -15,7 +15,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library links against)
 
 from ..csrc import build as _build
 
-ABI_VERSION = 20
+ABI_VERSION = 21
 
 
 class KernelLibraryError(RuntimeError):
@@ -53,7 +53,17 @@ _SIGNATURES = {
     "ra_stream_add": [P, P, I, P, P, I, I, I, F, P],
     "ra_tanh_cap": [P, I, I, I, F, P],
     "ra_latent_prep": [P, I, I, I, I, P, I, F, P, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
-    "ra_head_linear": [P, I, I, P, P, I, I, P, I, I, I, I, I, I, P],
+    "ra_head_linear": [P, I, I, P, P, I, I, P, I, I, I, I, I, I, I, P],
+    "ra_add_group_rmsnorm": [P, P, P, I, P, I, P, I, I, I, F, F, P],
+    "ra_act_mul": [P, P, I, I, I, I, I, P],
+    "ra_moe_silu_gate_scale_shared": [P, P, I, P, P, I, I, I, I, P, I, I, P],
+    "ra_moe_route_softmax": [P, I, I, I, I, I, P, F, P, P, I, P],
+    "ra_moe_identity_add": [P, I, P, I, I, P, P, I, I, I, I, P],
+    "ra_wkv_scan": [P, I, I, I, I, I, P, I, P, P, P, c_long, P, P, P, I, I, I, I, I, P, P],
+    "ra_token_shift": [P, I, P, I, I, P, c_long, c_long, P, P, P, P, P, I, I, I, I, I, I, P],
+    "ra_gated_stream_add": [P, P, I, I, P, I, P, I, I, I, P],
+    "ra_rows_rmsnorm": [P, I, P, I, P, I, I, I, I, F, P],
+    "ra_tanh_rows": [P, I, c_long, P],
     "ra_moe_topk": [P, I, I, I, P, P, I, P],
     "ra_moe_relu2_scale": [P, P, I, P, P, I, I, I, I, P],
     "ra_moe_up_chosen": [P, I, P, P, P, P, I, I, I, I, I, I, P],

@@ -72,7 +72,9 @@ class HipKernels:
 
     def add_rmsnorm(self, resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor,
                     eps: float, out: torch.Tensor, rows: Optional[torch.Tensor] = None,
-                    delta_scale: float = 1.0) -> None:
+                    delta_scale: float = 1.0, groups: int = 1) -> None:
+        """``groups`` > 1: the row is normed in that many equal consecutive parts, each over its own root mean
+        square."""
         _dev(resid, delta, weight, out, rows)
         h = resid.shape[-1]
         n = out.shape[0]
@@ -88,6 +90,13 @@ class HipKernels:
                 raise ValueError("add_rmsnorm: in-place form needs one output row per residual row")
         else:
             _int32(rows, "add_rmsnorm rows", n)
+        if groups != 1:
+            if groups < 1 or h % groups:
+                raise ValueError(f"add_rmsnorm: width {h} does not split into {groups} equal groups")
+            library.call("ra_add_group_rmsnorm", resid.data_ptr(), _ptr(delta), weight.data_ptr(),
+                         _tag(weight, "norm weight"), out.data_ptr(), _tag(out, "add_rmsnorm out"),
+                         _ptr(rows), n, h, int(groups), float(eps), float(delta_scale), _stream())
+            return
         library.call("ra_add_rmsnorm", resid.data_ptr(), _ptr(delta), weight.data_ptr(),
                      _tag(weight, "norm weight"), out.data_ptr(), _tag(out, "add_rmsnorm out"),
                      _ptr(rows), n, h, float(eps), float(delta_scale), _stream())
@@ -185,9 +194,11 @@ class HipKernels:
                      int(rotary_dim), int(rope_style), slots.data_ptr(), kcache.data_ptr(), vcache.data_ptr(),
                      kcache.shape[2] * 16, T, num_heads, num_kv_heads, head_dim, _stream())
 
-    def silu_mul(self, gate_up: torch.Tensor, out: torch.Tensor, group: int = 0) -> None:
-        """out = silu(gate) * up. ``group`` 0: gate_up is [gate | up]; ``group`` g > 0: runs of g
-        gate columns and g up columns alternate."""
+    GATE_ACTS = {"silu": 0, "gelu_tanh": 1}
+
+    def silu_mul(self, gate_up: torch.Tensor, out: torch.Tensor, group: int = 0, act: str = "silu") -> None:
+        """out = act(gate) * up, act "silu" or "gelu_tanh" (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))).
+        ``group`` 0: gate_up is [gate | up]; ``group`` g > 0: runs of g gate columns and g up columns alternate."""
         _dev(gate_up, out)
         T, I = out.shape
         if gate_up.shape != (T, 2 * I) or gate_up.dtype != out.dtype \
@@ -195,8 +206,10 @@ class HipKernels:
             raise ValueError(f"silu_mul: gate_up {tuple(gate_up.shape)} against out {tuple(out.shape)}")
         if group < 0 or (group > 0 and I % group != 0):
             raise ValueError(f"silu_mul: width {I} is not a whole number of runs of {group}")
-        library.call("ra_silu_mul", gate_up.data_ptr(), out.data_ptr(), _tag(out, "silu_mul"), T, I,
-                     int(group), _stream())
+        if act not in self.GATE_ACTS:
+            raise ValueError(f"silu_mul: activation {act!r}; built: {sorted(self.GATE_ACTS)}")
+        library.call("ra_act_mul", gate_up.data_ptr(), out.data_ptr(), _tag(out, "silu_mul"), T, I,
+                     int(group), self.GATE_ACTS[act], _stream())
 
     # ------------------------------------------------------------- attention
     SHORT_PORTION = 4     # portions up to this many tokens go token by token through the decode kernel
@@ -965,7 +978,7 @@ class HipKernels:
                      vcache.data_ptr(), kcache.shape[2] * 16, T, _stream())
 
     def head_linear(self, x: torch.Tensor, x_head: int, weight: torch.Tensor, out: torch.Tensor, o_head: int,
-                    gate: Optional[torch.Tensor] = None) -> None:
+                    gate: Optional[torch.Tensor] = None, gate_per_head: bool = False) -> None:
         """Products head by head: out[t, h * o_head + n] = sum_k x[t, h * x_head + k] * weight[h, n, k], times
         sigmoid(gate[t, h * N + n]) where a gate is given. ``x``, ``out`` and ``gate`` are 2-D with unit
         column stride (they may be column ranges of wider buffers); ``weight`` is [heads, N, K] contiguous.
@@ -980,17 +993,17 @@ class HipKernels:
                 raise ValueError(f"head_linear: {what} must be [T, *] rows of the weight's dtype with unit column stride")
         if x.shape[1] < (H - 1) * x_head + K or out.shape[1] < (H - 1) * o_head + N or o_head < N:
             raise ValueError(f"head_linear: x {tuple(x.shape)} / out {tuple(out.shape)} do not hold {H} heads of {K} / {N}")
-        if gate is not None and gate.shape[1] < H * N:
-            raise ValueError(f"head_linear: gate {tuple(gate.shape)}, expected [T, {H * N}]")
+        if gate is not None and gate.shape[1] < (H if gate_per_head else H * N):
+            raise ValueError(f"head_linear: gate {tuple(gate.shape)}, expected [T, {H if gate_per_head else H * N}]")
         library.call("ra_head_linear", x.data_ptr(), x.stride(0), int(x_head), weight.data_ptr(), out.data_ptr(),
                      out.stride(0), int(o_head), _ptr(gate), gate.stride(0) if gate is not None else 0,
-                     _tag(x, "head_linear"), T, H, N, K, _stream())
+                     1 if gate_per_head else 0, _tag(x, "head_linear"), T, H, N, K, _stream())
 
     # ------------------------------------------------------ recurrent mixers
-    _SCAN_KINDS = {"matrix_memory": 0, "delta_rule": 1}
+    _SCAN_KINDS = {"matrix_memory": 0, "delta_rule": 1, "wkv": 2}
 
     def scan_state_floats(self, kind: str, heads: int, key_dim: int, value_dim: int) -> int:
-        """Floats of a request's state slot that the scan kernel of ``kind`` ("matrix_memory", "delta_rule")
+        """Floats of a request's state slot that the scan kernel of ``kind`` ("matrix_memory", "delta_rule", "wkv")
         keeps for ``heads`` heads of [key_dim, value_dim], in the kernel's own layout."""
         n = int(library.load().ra_scan_state_floats(self._SCAN_KINDS[kind], int(heads), int(key_dim), int(value_dim)))
         if n < 0:
@@ -1085,6 +1098,92 @@ class HipKernels:
                      int(getattr(batch, "max_q_len", 0) or 0), int(heads), int(key_heads), int(key_dim), int(value_dim),
                      out.data_ptr(), _stream())
 
+    def wkv_scan(self, proj: torch.Tensor, r_off: int, k_off: int, v_off: int, decay: torch.Tensor, w0: torch.Tensor,
+                 u: torch.Tensor, state: torch.Tensor, batch, heads: int, dim: int, out: torch.Tensor) -> None:
+        """A per-head matrix state with a decay a key channel and token, from and into ``state`` [slots, floats]:
+        o = (S + diag(u) k v^T)^T r, then S <- diag(w) S + k v^T with w = exp(-exp(decay + w0)). ``proj`` [T, *]
+        holds r, k, v (heads x dim each) from the given columns; ``decay`` float32 [T, heads * dim] the decays'
+        pre-activations; ``w0`` and ``u`` float32 [heads * dim]; ``out`` float32 [T, heads * dim]."""
+        _dev(proj, decay, w0, u, state, out)
+        T = proj.shape[0]
+        n = heads * dim
+        self._check_scan("wkv_scan", state, batch, T)
+        if proj.dim() != 2 or proj.stride(1) != 1 or max(r_off, k_off, v_off) + n > proj.shape[1]:
+            raise ValueError(f"wkv_scan: rows of {tuple(proj.shape)} do not hold r, k, v at {r_off}, {k_off}, {v_off}")
+        if decay.dim() != 2 or decay.shape[0] != T or decay.shape[1] < n or decay.dtype != torch.float32 \
+                or decay.stride(1) != 1:
+            raise ValueError(f"wkv_scan: decay pre-activations are float32 [T, {n}]")
+        for v, what in ((w0, "w0"), (u, "u")):
+            if v.shape != (n,) or v.dtype != torch.float32 or not v.is_contiguous():
+                raise ValueError(f"wkv_scan: {what} is float32 [{n}]")
+        if out.shape != (T, n) or out.dtype != torch.float32 or not out.is_contiguous():
+            raise ValueError("wkv_scan: out is contiguous float32 [T, heads * dim]")
+        library.call("ra_wkv_scan", proj.data_ptr(), _tag(proj, "wkv_scan"), proj.stride(0), int(r_off), int(k_off),
+                     int(v_off), decay.data_ptr(), decay.stride(0), w0.data_ptr(), u.data_ptr(), state.data_ptr(),
+                     state.stride(0), batch.cu_tokens.data_ptr(), batch.state_slots.data_ptr(), batch.fresh.data_ptr(),
+                     batch.num_seqs, T, int(getattr(batch, "max_q_len", 0) or 0), int(heads), int(dim), out.data_ptr(),
+                     _stream())
+
+    # ------------------------------------------- the token before, gated adds
+    def token_shift(self, h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, keep_off: int, batch,
+                    out: torch.Tensor) -> None:
+        """out[t, j * width + e] = h[t, e] + (prev(t)[e] - h[t, e]) * mu[j, e]: every row mixed with the row of
+        the token before it, once for each row of ``mu`` [n_mix, width]. The row before a portion's first comes
+        from ``state`` [slots, floats] at ``keep_off`` (zeros at a request's start), which then takes the
+        portion's last row; the kept row is float and holds the activations' values exactly."""
+        _dev(h, mu, state, out)
+        T, width = h.shape
+        if mu.dim() != 2 or mu.shape[1] != width or not mu.is_contiguous():
+            raise ValueError(f"token_shift: factors {tuple(mu.shape)}, expected [mixes, {width}]")
+        n_mix = mu.shape[0]
+        if h.stride(1) != 1 or out.shape != (T, n_mix * width) or out.stride(1) != 1 or out.dtype != h.dtype:
+            raise ValueError(f"token_shift: out {tuple(out.shape)}, expected [{T}, {n_mix * width}] in the input's dtype")
+        if state.shape[1] < keep_off + width:
+            raise ValueError("token_shift: the state slot does not hold the kept row")
+        self._check_scan("token_shift", state, batch, T)
+        single = 1 if int(getattr(batch, "max_q_len", 0) or 0) == 1 else 0
+        library.call("ra_token_shift", h.data_ptr(), h.stride(0), mu.data_ptr(), _tag(mu, "token_shift factors"), n_mix,
+                     state.data_ptr(), state.stride(0), int(keep_off), batch.seq_of_token.data_ptr(),
+                     batch.cu_tokens.data_ptr(), batch.state_slots.data_ptr(), batch.fresh.data_ptr(), out.data_ptr(),
+                     out.stride(0), _tag(h, "token_shift"), batch.num_seqs, T, width, single, _stream())
+
+    def gated_stream_add(self, resid: torch.Tensor, gates: torch.Tensor, a: torch.Tensor,
+                         b: Optional[torch.Tensor] = None) -> None:
+        """resid += sigmoid(gates[:, :width]) * a + sigmoid(gates[:, width:2 width]) * b, element by element, in
+        float; ``gates`` holds the pre-activations, ``b`` may be None."""
+        _dev(resid, gates, a, b)
+        T, width = resid.shape
+        if resid.dtype != torch.float32 or not resid.is_contiguous():
+            raise TypeError("gated_stream_add: the residual stream is contiguous float32")
+        need = (2 if b is not None else 1) * width
+        if gates.dim() != 2 or gates.shape[0] != T or gates.shape[1] < need or gates.stride(1) != 1:
+            raise ValueError(f"gated_stream_add: gates {tuple(gates.shape)}, expected [{T}, >= {need}]")
+        for t in (a, b):
+            if t is not None and (t.shape != (T, width) or not t.is_contiguous()):
+                raise ValueError("gated_stream_add: addends are contiguous [T, width]")
+        library.call("ra_gated_stream_add", resid.data_ptr(), gates.data_ptr(), gates.stride(0), _tag(gates, "gates"),
+                     a.data_ptr(), _tag(a, "addend"), _ptr(b), _tag(b, "addend") if b is not None else 0, T, width,
+                     _stream())
+
+    def rows_rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor) -> None:
+        """out = x / sqrt(mean(x^2) + eps) * weight over rows of activations (either may be a column range of a
+        wider buffer); the sums are float."""
+        _dev(x, weight, out)
+        T, width = x.shape
+        if out.shape != (T, width) or out.dtype != x.dtype or x.stride(1) != 1 or out.stride(1) != 1:
+            raise ValueError(f"rows_rmsnorm: x {tuple(x.shape)} against out {tuple(out.shape)}")
+        if weight.shape != (width,) or not weight.is_contiguous():
+            raise ValueError(f"rows_rmsnorm: weight {tuple(weight.shape)}, expected [{width}]")
+        library.call("ra_rows_rmsnorm", x.data_ptr(), x.stride(0), weight.data_ptr(), _tag(weight, "norm weight"),
+                     out.data_ptr(), out.stride(0), _tag(x, "rows_rmsnorm"), T, width, float(eps), _stream())
+
+    def tanh_rows(self, x: torch.Tensor) -> None:
+        """x <- tanh(x), in place."""
+        _dev(x)
+        if not x.is_contiguous():
+            raise ValueError("tanh_rows: a contiguous tensor")
+        library.call("ra_tanh_rows", x.data_ptr(), _tag(x, "tanh_rows"), x.numel(), _stream())
+
     def head_norm_gate(self, read: torch.Tensor, weight: torch.Tensor, per_head: bool, gate: torch.Tensor, kind: str,
                        eps: float, heads: int, value_dim: int, out: torch.Tensor) -> None:
         """out[t, h] = read[t, h] / rms(read[t, h]) * weight * act(gate[t, h]) head by head: ``read`` float32
@@ -1136,13 +1235,18 @@ class HipKernels:
     # ---------------------------------------------------- mixture of experts
     def moe_route(self, x: torch.Tensor, router: torch.Tensor, top: int, ids: torch.Tensor,
                   weights: torch.Tensor, scoring: str = "softmax_chosen", scale: float = 1.0, groups: int = 1,
-                  groups_kept: int = 1, group_top: int = 2) -> None:
+                  groups_kept: int = 1, group_top: int = 2, correction: Optional[torch.Tensor] = None,
+                  norm_eps: float = 0.0, outputs: Optional[int] = None) -> torch.Tensor:
         """Router logits x . router^T accumulated and kept in float (``router`` [experts, width] in the
         activations' dtype: a bfloat16 product's terms are exact in float), the ``top`` largest a token in
         falling order into ``ids`` [T, top] (int32), the softmax over those alone into ``weights`` [T, top]
         (float32). ``scoring`` "sigmoid": scores are the logits' sigmoids; with ``groups`` > 1 only experts of
         the ``groups_kept`` best groups of neighbours (a group's score: the sum of its ``group_top`` largest
-        scores) can be chosen; the weights are the chosen scores times ``scale``."""
+        scores) can be chosen; the weights are the chosen scores times ``scale``. ``scoring`` "softmax": scores
+        are the softmax over all outputs, the choice is by score + ``correction`` (float32 [outputs] or None)
+        inside the best groups (a group's score: its largest choice score), the weights the chosen scores over
+        their sum + ``norm_eps``. ``outputs``: the router's first rows that are routed over (default: all);
+        further rows are logits for the caller, who gets the float32 logits [T, rows] back."""
         _dev(x, router, ids, weights)
         T, width = x.shape
         E = router.shape[0]
@@ -1154,21 +1258,36 @@ class HipKernels:
             raise ValueError(f"moe_route: ids int32 and weights float32, both [{T}, {top}]")
         logits = torch.empty((T, E), dtype=torch.float32, device=x.device)
         self.linear(x, router, logits)
+        if outputs is not None:
+            if not 0 < outputs <= E:
+                raise ValueError(f"moe_route: {outputs} routed outputs of {E} router rows")
+            E = int(outputs)
+        if scoring == "softmax":
+            if correction is not None:
+                _dev(correction)
+                if correction.shape != (E,) or correction.dtype != torch.float32 or not correction.is_contiguous():
+                    raise ValueError(f"moe_route: correction is float32 [{E}]")
+            library.call("ra_moe_route_softmax", logits.data_ptr(), logits.stride(0), E, int(top), int(groups),
+                         int(groups_kept), _ptr(correction), float(norm_eps), ids.data_ptr(), weights.data_ptr(), T,
+                         _stream())
+            return logits
         if scoring == "sigmoid":
             library.call("ra_moe_route_sigmoid", logits.data_ptr(), logits.stride(0), E, int(top), int(groups),
                          int(groups_kept), int(group_top), float(scale), ids.data_ptr(), weights.data_ptr(), T,
                          _stream())
-            return
+            return logits
         if scoring != "softmax_chosen":
             raise ValueError(f"moe_route: scoring {scoring!r}")
         library.call("ra_moe_topk", logits.data_ptr(), logits.stride(0), E, int(top), ids.data_ptr(),
                      weights.data_ptr(), T, _stream())
+        return logits
 
     def moe_silu_gate_scale(self, gu: torch.Tensor, act: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor,
-                            experts: int, ff: int, shared: int = 0) -> None:
+                            experts: int, ff: int, shared: int = 0, shared_logit: Optional[torch.Tensor] = None) -> None:
         """``gu`` [T, 2 (experts ff + shared)]: [gate | up] of each expert, a shared expert's behind them.
         act[t, e ff + j] = weight(t, e) silu(gate) up for the chosen experts, 0 for the others; the shared
-        expert's columns behind them with weight 1."""
+        expert's columns behind them with weight 1, or with sigmoid(``shared_logit``[t]) (float32, one number a
+        token; it may be a column of a wider matrix). A chosen id of ``experts`` or more names no matrices."""
         _dev(gu, act, ids, weights)
         T = gu.shape[0]
         n = experts * ff + shared
@@ -1177,8 +1296,27 @@ class HipKernels:
             raise ValueError(f"moe_silu_gate_scale: gu {tuple(gu.shape)} / act {tuple(act.shape)}, expected "
                              f"[T, {2 * n}] and [T, {n}]")
         self._check_choice("moe_silu_gate_scale", ids, weights, T, ids.shape[1])
-        library.call("ra_moe_silu_gate_scale", gu.data_ptr(), act.data_ptr(), _tag(gu, "moe_silu_gate_scale"),
-                     ids.data_ptr(), weights.data_ptr(), ids.shape[1], int(experts), int(ff), int(shared), T, _stream())
+        ld = 0
+        if shared_logit is not None:
+            _dev(shared_logit)
+            if shared_logit.dtype != torch.float32 or shared_logit.shape[0] != T or shared_logit.numel() != T:
+                raise ValueError("moe_silu_gate_scale: the shared expert's logits are float32, one a token")
+            ld = shared_logit.stride(0)
+        library.call("ra_moe_silu_gate_scale_shared", gu.data_ptr(), act.data_ptr(), _tag(gu, "moe_silu_gate_scale"),
+                     ids.data_ptr(), weights.data_ptr(), ids.shape[1], int(experts), int(ff), int(shared),
+                     _ptr(shared_logit), int(ld), T, _stream())
+
+    def moe_identity_add(self, y: torch.Tensor, x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor,
+                         experts: int) -> None:
+        """y[t] += (sum of weights[t, j] over choices with ids[t, j] >= experts) * x[t]: chosen ids past the
+        experts stand for the identity."""
+        _dev(y, x, ids, weights)
+        T, width = y.shape
+        if x.shape != (T, width) or x.dtype != y.dtype or x.stride(1) != 1 or y.stride(1) != 1:
+            raise ValueError(f"moe_identity_add: y {tuple(y.shape)} against x {tuple(x.shape)}")
+        self._check_choice("moe_identity_add", ids, weights, T, ids.shape[1])
+        library.call("ra_moe_identity_add", y.data_ptr(), y.stride(0), x.data_ptr(), x.stride(0), _tag(y, "moe_identity_add"),
+                     ids.data_ptr(), weights.data_ptr(), ids.shape[1], int(experts), T, width, _stream())
 
     def moe_relu2_scale(self, up: torch.Tensor, act: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor,
                         experts: int, ff: int) -> None:

@@ -15,8 +15,8 @@ from typing import Dict, List, Optional
 import torch
 
 from ..config.schema import BlockSpec
-from ..weights import ParamDecl
-from .base import LayerCache
+from ..weights import VECTOR, ParamDecl
+from .base import JointNeed, LayerCache, StateNeed
 from .registry import lookup, register_block
 
 
@@ -145,7 +145,19 @@ class ParallelBlock:
     """h = norm(x); x += mixer(h) + ffn(h): one norm, and both parts read its output. A block without a
     feed-forward (``spec.ffn`` None) is x += mixer(norm(x)). The sums are float: a part that can add its last
     product into the stream does so, any other addend goes through the stream-add kernel or, the last one,
-    back to the caller, whose next norm adds it."""
+    back to the caller, whose next norm adds it.
+
+    Two options (``spec.params``, a :class:`ParallelSpec`). ``token_shift``: the mixer reads
+    h + (h' - h) * s, h' being the normed row of the token before (zeros for a request's first token); the
+    feed-forward reads h as it is. The last h of a portion is kept in the request's state, so the layer's cache
+    is the mixer's and, beside it, one row of the width. ``gated``: x += sigmoid(W1 h + b1) * mixer(...) +
+    sigmoid(W2 h + b2) * ffn(h); both gates come from one product over h and the sum is one float kernel."""
+
+    @staticmethod
+    def _options(spec: BlockSpec):
+        o = spec.params
+        return (bool(getattr(o, "token_shift", False)), bool(getattr(o, "gated", False)),
+                str(getattr(o, "shift_name", "shift")), tuple(getattr(o, "gate_names", ("rg1", "rg2"))))
 
     @classmethod
     def declare_params(cls, spec: BlockSpec) -> List[ParamDecl]:
@@ -154,6 +166,13 @@ class ParallelBlock:
         out += lookup("mixer", spec.mixer.kind).declare_params(spec.mixer, p + spec.mixer_prefix)
         if spec.ffn is not None:
             out += lookup("feed_forward", spec.ffn.kind).declare_params(spec.ffn, p + spec.ffn_prefix)
+        shift, gated, shift_name, gate_names = cls._options(spec)
+        w = spec.mixer_norm.size
+        if shift:
+            out.append(ParamDecl(p + shift_name, (w,), role=VECTOR))
+        if gated:
+            for name in gate_names[:2 if spec.ffn is not None else 1]:
+                out += [ParamDecl(p + name, (w, w)), ParamDecl(p + name + ".b", (w,), init="zeros", role=VECTOR)]
         return out
 
     def __init__(self, spec: BlockSpec, weights: Dict[str, torch.Tensor], dtype: torch.dtype,
@@ -170,6 +189,16 @@ class ParallelBlock:
         self.ffn = None
         if spec.ffn is not None:
             self.ffn = lookup("feed_forward", spec.ffn.kind)(spec.ffn, weights, p + spec.ffn_prefix, dtype, device)
+        self.dtype = dtype
+        self.width = int(spec.mixer_norm.size)
+        self.token_shift, self.gated, shift_name, gate_names = self._options(spec)
+        if self.token_shift:
+            self.shift = weights[p + shift_name].to(dtype).view(1, self.width).contiguous()
+        if self.gated:
+            names = gate_names[:2 if self.ffn is not None else 1]
+            # both gates' pre-activations from one product over h: rows of the mixer's gate, then the feed-forward's
+            self.w_gates = torch.cat([weights[p + n] for n in names], dim=0).contiguous()
+            self.b_gates = torch.cat([weights[p + n + ".b"] for n in names], dim=0).to(self.w_gates.dtype).contiguous()
 
     @property
     def graph_safe(self) -> bool:
@@ -177,16 +206,42 @@ class ParallelBlock:
                     and (self.ffn is None or getattr(self.ffn, "graph_safe", False)))
 
     def cache_need(self):
-        return self.mixer.cache_need() if hasattr(self.mixer, "cache_need") else None
+        need = self.mixer.cache_need() if hasattr(self.mixer, "cache_need") else None
+        if self.token_shift:
+            # the mixer's own need and, beside it, the last normed row of the request
+            return JointNeed((need, StateNeed((self.width,), torch.float32)))
+        return need
 
     def parts(self):
         return tuple(p for p in (self.norm, self.mixer, self.ffn) if p is not None)
+
+    def _forward_shift_gate(self, resid: torch.Tensor, h: torch.Tensor, batch, cache: Optional[LayerCache]):
+        """The block with a token shift and / or gates on its addends: nothing is left pending."""
+        from .. import kernels
+        ops = kernels.current()
+        T = h.shape[0]
+        mixer_cache, hs = cache, h
+        if self.token_shift:
+            mixer_cache, kept = cache.members
+            hs = torch.empty_like(h)
+            ops.token_shift(h, self.shift, kept.state, 0, batch, hs)
+        a = self.mixer.forward(hs, batch, mixer_cache)
+        b = self.ffn.forward(h, batch) if self.ffn is not None else None
+        if self.gated:
+            gates = torch.empty((T, self.w_gates.shape[0]), dtype=self.dtype, device=h.device)
+            ops.linear(h, self.w_gates, gates, self.b_gates)
+            ops.gated_stream_add(resid, gates, a, b)
+            return None
+        ops.stream_add(resid, a)
+        return b
 
     def forward(self, resid: torch.Tensor, delta, batch, cache: Optional[LayerCache]):
         from .. import kernels
         if not isinstance(delta, torch.Tensor) and delta is not None:
             delta = None               # a filled norm target: the sum is already in the stream
         h = self.norm.add_norm(resid, delta)          # the stream now holds everything before this block
+        if self.token_shift or self.gated:
+            return self._forward_shift_gate(resid, h, batch, cache)
         addends = []
         if getattr(self.mixer, "adds_in_place", False):
             a = self.mixer.forward(h, batch, cache, resid=resid)

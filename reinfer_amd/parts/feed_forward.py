@@ -6,6 +6,8 @@ their rows are interleaved in runs of 8 at load (8 gate rows, the 8 up rows of
 the same features, ...), so that for few tokens the product's epilogue applies
 the gate itself and for many the gate kernel reads both from one cache line.
 A width that is no multiple of 8 keeps [gate; up] and the separate gate kernel.
+The option ``act`` names another gate activation ("gelu_tanh": 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))));
+it is applied by the gate kernel behind the product.
 """
 from __future__ import annotations
 
@@ -56,6 +58,9 @@ class SwiGLU:
             self.group = 0
             self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
         self.w_down = weights[prefix + dn]
+        self.act = str(dict(spec.extra).get("act", "silu"))
+        if self.act not in ("silu", "gelu_tanh"):
+            raise ValueError(f"swiglu: gate activation {self.act!r}; built: silu, gelu_tanh")
 
     def forward(self, x, batch, resid: Optional[torch.Tensor] = None, emit: Optional[NormTarget] = None,
                 resid_scale: float = 1.0):
@@ -64,7 +69,15 @@ class SwiGLU:
         T = x.shape[0]
         I = self.spec.intermediate
         act = torch.empty((T, I), dtype=self.dtype, device=x.device)
-        if self.group:
+        if self.act != "silu":
+            # the products' gated epilogue is silu: another activation runs as the gate kernel
+            gu = torch.empty((T, 2 * I), dtype=self.dtype, device=x.device)
+            if row_sums is None:
+                ops.linear(x, self.w_gate_up, gu)
+            else:
+                ops.linear_skinny(x, self.w_gate_up, gu, row_sums=row_sums)
+            ops.silu_mul(gu, act, self.group, act=self.act)
+        elif self.group:
             if row_sums is None:
                 ops.gated_linear(x, self.w_gate_up, act)
             else:

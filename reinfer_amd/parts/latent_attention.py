@@ -15,6 +15,10 @@ kernels as grouped-query attention: queries [W_uk,a^T q_a | rot(qr_a)], values t
 behind ``rank`` of the result are not used). What is new here are the kernel that norms, rotates and writes
 the cache row (``latent_prep``) and the products head by head before and after (``head_linear``).
 q, the latent and the gate come from one fused product.
+
+Two options. ``q_rank`` > 0: the queries come through a latent of their own, q = W_uq (rms(W_dq h) * w_q): the
+fused product then makes [latent of q | latent | key part | gate], a row norm and a second product make q.
+``head_gate``: the gate is one number a head, sigmoid(W_g h)_a with W_g [heads, width], not one a value entry.
 """
 from __future__ import annotations
 
@@ -42,13 +46,18 @@ class LatentAttention:
     def declare_params(cls, spec: MixerSpec, prefix: str) -> List[ParamDecl]:
         p = spec.params
         H, D, R = spec.num_heads, spec.head_dim, p.rot_width
-        out = [ParamDecl(prefix + "q", (H * (D + R), spec.hidden)),
-               ParamDecl(prefix + "dkv", (p.rank + R, spec.hidden)),
+        if p.q_rank:
+            out = [ParamDecl(prefix + "dq", (p.q_rank, spec.hidden)),
+                   ParamDecl(prefix + "dq.norm", (p.q_rank,), init="norm", role=VECTOR),
+                   ParamDecl(prefix + "uq", (H * (D + R), p.q_rank))]
+        else:
+            out = [ParamDecl(prefix + "q", (H * (D + R), spec.hidden))]
+        out += [ParamDecl(prefix + "dkv", (p.rank + R, spec.hidden)),
                ParamDecl(prefix + "dkv.norm", (p.rank,), init="norm", role=VECTOR),
                ParamDecl(prefix + "uk", (H * D, p.rank)),
                ParamDecl(prefix + "uv", (H * p.value_dim, p.rank))]
         if p.gated:
-            out.append(ParamDecl(prefix + "g", (H * p.value_dim, spec.hidden)))
+            out.append(ParamDecl(prefix + "g", (H if p.head_gate else H * p.value_dim, spec.hidden)))
         out.append(ParamDecl(prefix + "o", (spec.hidden, H * p.value_dim)))
         return out
 
@@ -62,22 +71,48 @@ class LatentAttention:
         self.num_heads, self.head_dim = int(spec.num_heads), int(spec.head_dim)
         self.rank, self.rot_width, self.value_dim = int(p.rank), int(p.rot_width), int(p.value_dim)
         self.gated = bool(p.gated)
+        self.head_gate = bool(p.head_gate)
+        self.q_rank = int(p.q_rank)
         self.eps = float(p.norm_eps)
         self.scale = float(spec.scale)
         self.window = int(spec.window)
         self.cache_dim = _round16(self.rank + self.rot_width)
         H, D, R, Dv = self.num_heads, self.head_dim, self.rot_width, self.value_dim
-        # one product for everything that reads the mixer's input: rows of q, of the latent, of the gate
-        rows = [weights[prefix + "q"], weights[prefix + "dkv"]]
-        self.q_off, self.dkv_off = 0, H * (D + R)
-        self.gate_off = self.dkv_off + self.rank + R
+        # one product for everything that reads the mixer's input: rows of q (or of its latent), of the latent,
+        # of the gate. The buffer's row always starts with the H query heads, which a second product fills
+        # where the queries go through a latent of their own; every part starts at a multiple of 8 columns
+        # (16-byte pieces for the kernels that read them).
+        def pad8(n: int) -> int:
+            return -(-n // 8) * 8
+
+        def zeros(n: int):
+            return torch.zeros((n, spec.hidden), dtype=self.w_dtype, device=weights[prefix + "dkv"].device)
+        self.w_dtype = weights[prefix + "dkv"].dtype
+        self.gate_width = (H if self.head_gate else H * Dv) if self.gated else 0
+        self.q_off = 0
+        self.dkv_off = pad8(H * (D + R))
+        self.gate_off = self.dkv_off + pad8(self.rank + R)
+        self.dq_off = self.gate_off + pad8(self.gate_width)
+        self.proj_width = self.dq_off + pad8(self.q_rank)
+        parts = [(self.dkv_off, weights[prefix + "dkv"])]
         if self.gated:
-            rows.append(weights[prefix + "g"])
-        self.proj_width = sum(int(w.shape[0]) for w in rows)
-        pad = (-self.proj_width) % 8            # rows of 16-byte pieces for the kernels that read them
-        if pad:
-            rows.append(torch.zeros((pad, spec.hidden), dtype=rows[0].dtype, device=rows[0].device))
-        self.proj_width += pad
+            parts.append((self.gate_off, weights[prefix + "g"]))
+        if self.q_rank:
+            parts.append((self.dq_off, weights[prefix + "dq"]))
+            self.in_off = self.dkv_off          # the fused product fills the row from here on
+            self.w_uq = weights[prefix + "uq"]
+            self.q_norm = weights[prefix + "dq.norm"]
+        else:
+            parts.insert(0, (0, weights[prefix + "q"]))
+            self.in_off = 0
+        rows, at = [], self.in_off
+        for off, w in parts:
+            if off > at:
+                rows.append(zeros(off - at))
+            rows.append(w)
+            at = off + int(w.shape[0])
+        if self.proj_width > at:
+            rows.append(zeros(self.proj_width - at))
         self.w_in = torch.cat(rows, dim=0).contiguous()
         self.c_norm = weights[prefix + "dkv.norm"]
         # head products, [heads, N, K] with K contiguous: queries through the key matrices, W_uk[a, d, r] transposed
@@ -126,7 +161,12 @@ class LatentAttention:
         H, D, Dv, Dp = self.num_heads, self.head_dim, self.value_dim, self.cache_dim
         slots = batch.slots[cache.group] if cache.writes else batch.no_slots
         proj = torch.empty((T, self.proj_width), dtype=self.dtype, device=x.device)
-        ops.linear(x, self.w_in, proj)
+        ops.linear(x, self.w_in, proj[:, self.in_off:])
+        if self.q_rank:
+            # the queries' latent, normed in float over its own width, then up to the heads
+            cq = torch.empty((T, self.q_rank), dtype=self.dtype, device=x.device)
+            ops.rows_rmsnorm(proj[:, self.dq_off:self.dq_off + self.q_rank], self.q_norm, self.eps, cq)
+            ops.linear(cq, self.w_uq, proj[:, :H * (D + self.rot_width)])
         q_lat = torch.empty((T, H, Dp), dtype=self.dtype, device=x.device)
         ops.latent_prep(proj, self.q_off, self.dkv_off, self.c_norm, self.eps, batch.positions,
                         self.position.inv_freq, self.position.rotary_dim, self.rot_width, self.rank, H, D,
@@ -143,7 +183,8 @@ class LatentAttention:
                           Dp, self.scale, self.window, cache.group)
         heads = torch.empty((T, H * Dv), dtype=self.dtype, device=x.device)
         ops.head_linear(o_lat, Dp, self.w_values, heads, Dv,
-                        gate=proj[:, self.gate_off:self.gate_off + H * Dv] if self.gated else None)
+                        gate=proj[:, self.gate_off:self.gate_off + self.gate_width] if self.gated else None,
+                        gate_per_head=self.head_gate)
         can_add = getattr(ops, "can_accumulate", None)
         if resid is not None and can_add and can_add(heads, self.w_o):
             ops.linear_skinny(heads, self.w_o, resid, accumulate=True)

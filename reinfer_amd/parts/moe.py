@@ -20,6 +20,13 @@ a shared expert of the same form may run for every token. Here every expert's [g
 after the other in one matrix, the shared expert's behind them, one kernel applies the gate and the
 routing weight (1 for the shared expert, 0 for experts not chosen), and one product with all down
 projections side by side is the sum.
+
+A third form (``activation`` "silu_gated", ``weights`` "softmax"): scores are the softmax of the router's logits
+over all its outputs; the choice is by score + a stored correction, inside the best groups (a group's score is
+its largest choice score); the weights are the chosen scores over their sum. The router's last ``identity``
+outputs stand for experts without matrices whose output is the token's input row; the shared expert's result is
+multiplied by the sigmoid of one more logit a token (its weight row lies behind the router's, so the same float
+product makes it). The experts' matrices and the two products are those of the second form.
 """
 from __future__ import annotations
 
@@ -29,7 +36,7 @@ import torch
 
 from .. import kernels
 from ..config.schema import FeedForwardSpec
-from ..weights import ParamDecl
+from ..weights import VECTOR, ParamDecl
 from .registry import register_feed_forward
 
 
@@ -49,12 +56,16 @@ class MixtureOfExperts:
                 out.append(ParamDecl(f"{prefix}e{e}.gate", (spec.intermediate, spec.hidden)))
             out += [ParamDecl(f"{prefix}e{e}.up", (spec.intermediate, spec.hidden)),
                     ParamDecl(f"{prefix}e{e}.down", (spec.hidden, spec.intermediate))]
-        out.append(ParamDecl(prefix + "router", (p.experts, spec.hidden)))
+        out.append(ParamDecl(prefix + "router", (p.experts + p.identity, spec.hidden)))
+        if p.correction:
+            out.append(ParamDecl(prefix + "correction", (p.experts + p.identity,), init="zeros", role=VECTOR))
         if p.shared:
             if gated:
                 out.append(ParamDecl(prefix + "shared.gate", (p.shared, spec.hidden)))
             out += [ParamDecl(prefix + "shared.up", (p.shared, spec.hidden)),
                     ParamDecl(prefix + "shared.down", (spec.hidden, p.shared))]
+            if p.shared_gated:
+                out.append(ParamDecl(prefix + "shared.sg", (1, spec.hidden)))
         return out
 
     def __init__(self, spec: FeedForwardSpec, weights: Dict[str, torch.Tensor], prefix: str,
@@ -62,20 +73,34 @@ class MixtureOfExperts:
         p = spec.params
         if p is None:
             raise ValueError("moe: the routing comes in FeedForwardSpec.params (MoESpec)")
-        if (p.activation, p.weights) not in (("relu2", "softmax_chosen"), ("silu_gated", "sigmoid")):
+        if (p.activation, p.weights) not in (("relu2", "softmax_chosen"), ("silu_gated", "sigmoid"),
+                                             ("silu_gated", "softmax")):
             raise ValueError(f"moe: activation {p.activation!r} with weights {p.weights!r} is not built")
         self.spec = spec
         self.dtype = dtype
         self.experts, self.top, self.ff = int(p.experts), int(p.top), int(spec.intermediate)
         self.gated = p.activation == "silu_gated"
         self.routing = p
-        if p.groups < 1 or p.experts % p.groups or not 1 <= p.groups_kept <= p.groups \
-                or p.top > p.groups_kept * (p.experts // p.groups):
-            raise ValueError(f"moe: {p.experts} experts in {p.groups} groups of which {p.groups_kept} are kept "
+        self.identity = int(p.identity)
+        routed = self.experts + self.identity             # groups are formed over experts and identity experts together
+        if p.groups < 1 or routed % p.groups or not 1 <= p.groups_kept <= p.groups \
+                or p.top > p.groups_kept * (routed // p.groups):
+            raise ValueError(f"moe: {routed} experts in {p.groups} groups of which {p.groups_kept} are kept "
                              f"cannot give {p.top} choices")
+        if p.weights != "softmax" and (p.identity or p.correction or p.shared_gated):
+            raise ValueError("moe: identity experts, a correction of the choice and a gate on the shared expert "
+                             "are built for the softmax router")
+        if p.weights == "softmax" and p.groups > 1 and p.group_top != 1:
+            raise ValueError("moe: the softmax router scores a group by its largest choice score (group_top 1)")
+        if p.shared_gated and not p.shared:
+            raise ValueError("moe: a gate on the shared expert needs a shared expert")
         if (p.groups > 1 or p.shared) and not self.gated:
             raise ValueError("moe: groups of experts and a shared expert are built for the gated form")
         self.router = weights[prefix + "router"]            # logits are accumulated and kept in float
+        self.correction = weights[prefix + "correction"].float().contiguous() if p.correction else None
+        if p.shared_gated:
+            # the shared expert's gate is one more row of the float product that makes the router's logits
+            self.router = torch.cat([self.router, weights[prefix + "shared.sg"]], dim=0).contiguous()
         if self.gated:
             self.shared = int(p.shared)
             rows = []
@@ -98,12 +123,30 @@ class MixtureOfExperts:
         n = self.experts * self.ff + self.shared
         ids = torch.empty((T, self.top), dtype=torch.int32, device=x.device)
         weights = torch.empty((T, self.top), dtype=torch.float32, device=x.device)
-        ops.moe_route(x, self.router, self.top, ids, weights, scoring="sigmoid", scale=float(p.weight_scale),
-                      groups=int(p.groups), groups_kept=int(p.groups_kept), group_top=int(p.group_top))
+        routed = self.experts + self.identity
+        shared_logit = None
+        if p.weights == "softmax":
+            logits = ops.moe_route(x, self.router, self.top, ids, weights, scoring="softmax", groups=int(p.groups),
+                                   groups_kept=int(p.groups_kept), correction=self.correction,
+                                   norm_eps=float(p.norm_eps), outputs=routed)
+            if p.shared_gated:
+                shared_logit = logits[:, routed]
+        else:
+            ops.moe_route(x, self.router, self.top, ids, weights, scoring="sigmoid", scale=float(p.weight_scale),
+                          groups=int(p.groups), groups_kept=int(p.groups_kept), group_top=int(p.group_top))
         gu = torch.empty((T, 2 * n), dtype=self.dtype, device=x.device)
         ops.linear(x, self.w_gate_up, gu)
         act = torch.empty((T, n), dtype=self.dtype, device=x.device)
-        ops.moe_silu_gate_scale(gu, act, ids, weights, self.experts, self.ff, self.shared)
+        if shared_logit is not None:
+            ops.moe_silu_gate_scale(gu, act, ids, weights, self.experts, self.ff, self.shared, shared_logit=shared_logit)
+        else:
+            ops.moe_silu_gate_scale(gu, act, ids, weights, self.experts, self.ff, self.shared)
+        if self.identity:
+            # the chosen identity experts' share, weight times the input row, is added to the product's result
+            out = torch.empty((T, self.spec.hidden), dtype=self.dtype, device=x.device)
+            ops.linear(act, self.w_down, out)
+            ops.moe_identity_add(out, x, ids, weights, self.experts)
+            return out
         can_add = getattr(ops, "can_accumulate", None)
         if resid is not None and can_add and can_add(act, self.w_down):
             if resid_scale != 1.0:

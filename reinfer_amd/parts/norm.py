@@ -1,7 +1,8 @@
 """RMSNorm, alone and fused with the residual add.
 
 y = x * rsqrt(mean(x^2) + eps) * w, eps inside the root
-(crates/cuda/kernels/dense_kernels.cu:59-88; crates/kernels/src/refs.rs:10-18).
+(crates/cuda/kernels/dense_kernels.cu:59-88; crates/kernels/src/refs.rs:10-18). With ``groups`` > 1 the
+row is split into that many equal consecutive parts and each is divided by its own root mean square.
 """
 from __future__ import annotations
 
@@ -26,6 +27,9 @@ class RMSNorm:
                  dtype: torch.dtype, device: torch.device):
         self.size = spec.size
         self.eps = float(spec.eps)
+        self.groups = int(getattr(spec, "groups", 1) or 1)
+        if self.groups < 1 or spec.size % self.groups:
+            raise ValueError(f"rmsnorm: width {spec.size} does not split into {self.groups} equal groups")
         self.weight = weights[name]
         if spec.offset:
             # a weight stored around zero: the factor offset + w is made once, in float
@@ -51,7 +55,10 @@ class RMSNorm:
             delta = None
         n = resid.shape[0] if rows is None else rows.numel()
         out = torch.empty((n, self.size), dtype=self.dtype, device=resid.device)
-        if delta is not None and delta_scale != 1.0:
+        if self.groups != 1:
+            kernels.current().add_rmsnorm(resid, delta, self.weight, self.eps, out, rows,
+                                          delta_scale=float(delta_scale), groups=self.groups)
+        elif delta is not None and delta_scale != 1.0:
             kernels.current().add_rmsnorm(resid, delta, self.weight, self.eps, out, rows, delta_scale=float(delta_scale))
         else:
             kernels.current().add_rmsnorm(resid, delta, self.weight, self.eps, out, rows)
@@ -67,7 +74,8 @@ class RMSNorm:
         T = resid.shape[0]
         # the product behind this norm reads rows of this width as 16-byte pieces: a width that is no
         # multiple of 8 goes through the norm kernel and the plain product
-        if parts is None or self.dtype != torch.bfloat16 or resid.shape[1] != self.size or self.size % 8 != 0:
+        if parts is None or self.dtype != torch.bfloat16 or resid.shape[1] != self.size or self.size % 8 != 0 \
+                or self.groups != 1:          # the hand-over carries one row factor: a norm in groups has several
             return None
         few = getattr(ops, "NORM_ON_PRODUCTS_ROWS", 0)
         if few < T <= getattr(ops, "NORM_FINISHED_ROWS", 0):

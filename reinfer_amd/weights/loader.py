@@ -139,6 +139,17 @@ def load_weights(model_dir: str, decls: Sequence[ParamDecl], compute_dtype: torc
             f.close()
 
 
+def tensor_shapes(model_dir: str) -> Dict[str, Tuple[int, ...]]:
+    """name -> shape of every tensor of a model folder, from the files' headers alone (no data is read): for a
+    configuration some of whose sizes only the tensors give."""
+    files, where = _open_folder(model_dir)
+    try:
+        return {n: tuple(files[f].shape(n)) for n, f in where.items() if n in files[f].entries}
+    finally:
+        for f in files.values():
+            f.close()
+
+
 def weight_from_folder(model_dir: str, name: str) -> torch.Tensor:
     """One tensor of a model folder, as stored, on the CPU."""
     files, where = _open_folder(model_dir)

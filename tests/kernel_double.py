@@ -30,7 +30,7 @@ class KernelDouble:
     def embed(self, table, ids, out, scale=1.0):
         out.copy_(table[ids.long()].float() * scale)
 
-    def add_rmsnorm(self, resid, delta, weight, eps, out, rows=None, delta_scale=1.0):
+    def add_rmsnorm(self, resid, delta, weight, eps, out, rows=None, delta_scale=1.0, groups=1):
         if rows is None:
             if delta is not None:
                 resid.add_(delta.float() * delta_scale)
@@ -39,8 +39,10 @@ class KernelDouble:
             x = resid[rows.long()]
             if delta is not None:
                 x = x + delta[rows.long()].float() * delta_scale
-        rstd = torch.rsqrt((x * x).mean(dim=-1, keepdim=True) + eps)
-        out.copy_((x * rstd * weight.float()).to(out.dtype))
+        n, h = x.shape
+        xg = x.view(n, groups, h // groups)
+        rstd = torch.rsqrt((xg * xg).mean(dim=-1, keepdim=True) + eps)
+        out.copy_(((xg * rstd).reshape(n, h) * weight.float()).to(out.dtype))
 
     def qk_norm_rope_cache(self, qkv, q_weight, k_weight, eps, positions, inv_freq, rotary_dim,
                            rope_style, slots, kcache, vcache, num_heads, num_kv_heads, head_dim):
@@ -152,18 +154,18 @@ class KernelDouble:
             kflat[s // bs][:, k_index(s % bs, e, Dp)] = row[t].to(kcache.dtype)
             vflat[s // bs][:, v_index(s % bs, e, Dp)] = row[t].to(vcache.dtype)
 
-    def head_linear(self, x, x_head, weight, out, o_head, gate=None):
+    def head_linear(self, x, x_head, weight, out, o_head, gate=None, gate_per_head=False):
         H, N, K = weight.shape
         for h in range(H):
             y = x[:, h * x_head:h * x_head + K].float() @ weight[h].float().T
             if gate is not None:
-                y = y * torch.sigmoid(gate[:, h * N:(h + 1) * N].float())
+                y = y * torch.sigmoid((gate[:, h:h + 1] if gate_per_head else gate[:, h * N:(h + 1) * N]).float())
             out[:, h * o_head:h * o_head + N] = y.to(out.dtype)
 
     # ---- recurrent mixers (state in a layout of this stand-in's own: the state is the kernels' private matter)
     @staticmethod
     def scan_state_floats(kind, heads, key_dim, value_dim):
-        return heads * key_dim * value_dim + (heads * (key_dim + 1) if kind == "matrix_memory" else 0)
+        return heads * key_dim * value_dim + (heads * (key_dim + 1) if kind == "matrix_memory" else 0)   # "delta_rule", "wkv": S alone
 
     @staticmethod
     def _requests(batch):
@@ -248,6 +250,52 @@ class KernelDouble:
                 S.add_(k[:, :, None] * u[:, None, :])
                 out[t] = torch.einsum("hkv,hk->hv", S, q).reshape(-1)
 
+    def wkv_scan(self, proj, r_off, k_off, v_off, decay, w0, u, state, batch, H, d, out):
+        p = proj.float()
+        w = torch.exp(-torch.exp(decay[:, :H * d] + w0)).view(-1, H, d)
+        uu = u.view(H, d)
+        for first, rows, slot, fresh in self._requests(batch):
+            if slot < 0:
+                out[first:first + rows] = 0
+                continue
+            S = state[slot, :H * d * d].view(H, d, d)
+            if fresh:
+                S.zero_()
+            for t in range(first, first + rows):
+                r = p[t, r_off:r_off + H * d].view(H, d)
+                k = p[t, k_off:k_off + H * d].view(H, d)
+                v = p[t, v_off:v_off + H * d].view(H, d)
+                kv = k[:, :, None] * v[:, None, :]
+                out[t] = torch.einsum("hkv,hk->hv", S + uu[:, :, None] * kv, r).reshape(-1)
+                S.mul_(w[t][:, :, None]).add_(kv)
+
+    # ---- the token before, gated adds, row norms
+    def token_shift(self, h, mu, state, keep_off, batch, out):
+        T, width = h.shape
+        x = h.float()
+        for first, rows, slot, fresh in self._requests(batch):
+            kept = state[slot, keep_off:keep_off + width] if slot >= 0 else None
+            before = torch.zeros(width) if (kept is None or fresh) else kept.clone()
+            prev = torch.cat([before[None, :], x[first:first + rows - 1]], dim=0)
+            cur = x[first:first + rows]
+            for j in range(mu.shape[0]):
+                out[first:first + rows, j * width:(j + 1) * width] = (cur + (prev - cur) * mu[j].float()).to(out.dtype)
+            if kept is not None:
+                kept.copy_(cur[-1])
+
+    def gated_stream_add(self, resid, gates, a, b=None):
+        width = resid.shape[1]
+        resid.add_(torch.sigmoid(gates[:, :width].float()) * a.float())
+        if b is not None:
+            resid.add_(torch.sigmoid(gates[:, width:2 * width].float()) * b.float())
+
+    def rows_rmsnorm(self, x, weight, eps, out):
+        v = x.float()
+        out.copy_((v * torch.rsqrt((v * v).mean(-1, keepdim=True) + eps) * weight.float()).to(out.dtype))
+
+    def tanh_rows(self, x):
+        x.copy_(torch.tanh(x.float()).to(x.dtype))
+
     def normed_mean(self, outs, weights, eps, out=None, resid=None, scale=1.0):
         y = 0
         for o, w in zip(outs, weights):
@@ -261,13 +309,29 @@ class KernelDouble:
 
     # ---- mixture of experts
     def moe_route(self, x, router, top, ids, weights, scoring="softmax_chosen", scale=1.0, groups=1, groups_kept=1,
-                  group_top=2):
-        z = x.float() @ router.float().T
+                  group_top=2, correction=None, norm_eps=0.0, outputs=None):
+        logits = x.float() @ router.float().T
+        z = logits if outputs is None else logits[:, :outputs]
         if scoring == "softmax_chosen":
             val, idx = torch.topk(z, top, dim=-1)
             ids.copy_(idx.to(torch.int32))
             weights.copy_(torch.softmax(val, dim=-1))
-            return
+            return logits
+        if scoring == "softmax":
+            s = torch.softmax(z, dim=-1)
+            c = s + correction if correction is not None else s.clone()
+            T, E = s.shape
+            if groups > 1:
+                gscore = c.view(T, groups, E // groups).max(-1).values
+                kept = torch.topk(gscore, groups_kept, dim=-1).indices
+                mask = torch.zeros(T, groups, dtype=torch.bool).scatter_(1, kept, True)
+                c = torch.where(mask[:, :, None].expand(T, groups, E // groups).reshape(T, E), c,
+                                torch.full_like(c, float("-inf")))
+            idx = torch.topk(c, top, dim=-1).indices
+            val = torch.gather(s, 1, idx)
+            ids.copy_(idx.to(torch.int32))
+            weights.copy_(val / (val.sum(-1, keepdim=True) + norm_eps))
+            return logits
         s = torch.sigmoid(z)
         T, E = s.shape
         allowed = s
@@ -281,16 +345,23 @@ class KernelDouble:
         val, idx = torch.topk(allowed, top, dim=-1)
         ids.copy_(idx.to(torch.int32))
         weights.copy_(val * scale)
+        return logits
 
-    def moe_silu_gate_scale(self, gu, act, ids, weights, experts, ff, shared):
+    def moe_identity_add(self, y, x, ids, weights, experts):
+        coef = (weights * (ids >= experts)).sum(-1, keepdim=True)
+        y.copy_((y.float() + coef * x.float()).to(y.dtype))
+
+    def moe_silu_gate_scale(self, gu, act, ids, weights, experts, ff, shared, shared_logit=None):
         T = gu.shape[0]
-        p = torch.zeros((T, experts))
+        p = torch.zeros((T, max(experts, int(ids.max()) + 1)))
         p.scatter_(1, ids.long(), weights)
+        p = p[:, :experts]
         g = gu[:, :2 * experts * ff].float().view(T, experts, 2, ff)
         a = (g[:, :, 0] * torch.sigmoid(g[:, :, 0]) * g[:, :, 1] * p[:, :, None]).reshape(T, experts * ff)
         if shared:
             sg = gu[:, 2 * experts * ff:].float().view(T, 2, shared)
-            a = torch.cat([a, sg[:, 0] * torch.sigmoid(sg[:, 0]) * sg[:, 1]], dim=1)
+            sw = torch.sigmoid(shared_logit.float())[:, None] if shared_logit is not None else 1.0
+            a = torch.cat([a, sw * sg[:, 0] * torch.sigmoid(sg[:, 0]) * sg[:, 1]], dim=1)
         act.copy_(a.to(act.dtype))
 
     def moe_relu2_scale(self, up, act, ids, weights, experts, ff):
@@ -323,14 +394,18 @@ class KernelDouble:
 
     GATE_GROUP = 8
 
-    def silu_mul(self, gate_up, out, group=0):
+    def silu_mul(self, gate_up, out, group=0, act="silu"):
         T, I = out.shape
         if group:
             v = gate_up.view(T, I // group, 2, group).float()
             g, u = v[:, :, 0].reshape(T, I), v[:, :, 1].reshape(T, I)
         else:
             g, u = gate_up[:, :I].float(), gate_up[:, I:].float()
-        out.copy_((g / (1 + torch.exp(-g)) * u).to(out.dtype))
+        if act == "gelu_tanh":
+            a = 0.5 * g * (1 + torch.tanh(0.7978845608028654 * (g + 0.044715 * g ** 3)))
+        else:
+            a = g / (1 + torch.exp(-g))
+        out.copy_((a * u).to(out.dtype))
 
     def gated_linear(self, x, weight, out, row_sums=None):
         gu = torch.empty((x.shape[0], weight.shape[0]), dtype=torch.float32)
