@@ -427,8 +427,66 @@ def kobolix_sizes():
     return out
 
 
+# ---------------------------------------------------------------------------------------------------
+# --design detatar: the Detatar design beside the Puresun design (the closest of the others: one norm for both
+# parts of a layer, attention over a cached latent, a mixture of experts) at equal size
+# ---------------------------------------------------------------------------------------------------
+def _detatar_raw(width, vocab, pattern, heads, kv_rank, q_rank, wkv_heads, dense_ff, moe):
+    """``pattern``: a string of layer codes: A attention + dense, a attention + experts, w wkv + experts,
+    r the wkv layer before it run again on its tensors."""
+    latent = {"dim": 128, "heads": heads, "kv_rank": kv_rank, "q_rank": q_rank, "rot": {"base": 1000000.0, "dims": 64},
+              "rot_dim": 64, "scale": 192 ** -0.5, "vdim": 128}
+    wkv = {"dim": 64, "heads": wkv_heads}
+    dense = {"ff": dense_ff, "kind": "dense"}
+    experts = {"expert": {"ff": moe[2]}, "kind": "moe", "shared": {"ff": moe[3]},
+               "router": {"experts": moe[0] - 2, "groups": {"count": 4, "keep": 2}, "identity": 2, "top": moe[1]}}
+    layers = []
+    for c in pattern:
+        if c == "r":
+            j = max(i for i, L in enumerate(layers) if L["type"] == "wkv" and "weights_of" not in L)
+            layers.append(dict(layers[j], weights_of=j))
+        else:
+            layers.append({"type": "wkv" if c == "w" else "latent_attention", "mixer": wkv if c == "w" else latent,
+                           "mlp": dense if c == "A" else experts})
+    return {"architecture": "Detatar", "vocab": vocab, "width": width, "norm": {"eps": 1e-5, "groups": 4},
+            "embedding": {"scale": 3.0}, "layers": layers,
+            "decay_ranks": [64 if L["type"] == "wkv" and "weights_of" not in L else 0 for L in layers]}
+
+
+def _parameters(raw) -> int:
+    import math
+    from reinfer_amd.config import config_from_dict
+    from reinfer_amd.models import declare_params
+    return sum(math.prod(p.shape) for p in declare_params(config_from_dict(raw).to_spec()) if not p.optional)
+
+
+# (name, Detatar configuration, its Puresun twin, vocabulary, "puresun"): as many layer runs, the same width, heads
+# and latent; the width of the twin's experts (a multiple of 64) is the one that brings its parameter count closest
+# to Detatar's
+def detatar_sizes():
+    out = []
+    for name, width, heads, q_rank, wkv_heads, dense_ff, moe in (
+            ("w2048", 2048, 16, 768, 32, 5632, (16, 4, 512, 1024)),
+            ("w4096", 4096, 16, 1536, 64, 11008, (16, 4, 1024, 2048))):
+        vocab, pattern = 32768, "Aawaar"
+        mixer = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 192, "scale": 192 ** -0.5,
+                 "rot": {"base": 1000000.0, "dims": 64}}
+
+        def twin(tff):
+            return {"architecture": "Puresun", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+                    "layers": [{"type": "latent_attention", "mixer": mixer,
+                                "mlp": {"kind": "moe", "expert": {"ff": tff}, "router": {"experts": moe[0], "top": moe[1]}}}
+                               for _ in pattern]}
+        raw = _detatar_raw(width, vocab, pattern, heads, 192, q_rank, wkv_heads, dense_ff, moe)
+        # the twin's count is linear in its experts' width
+        want, a, b = _parameters(raw), _parameters(twin(64)), _parameters(twin(128))
+        tff = max(64, round((64 + (want - a) * 64 / (b - a)) / 64) * 64)
+        out.append((name, raw, twin(tff), vocab, "puresun"))
+    return out
+
+
 def design_run(args) -> int:
-    """Prefill and decode throughput of the design (``--design``) and of its Qwen3 twin at each size, and the GPU time of a
+    """Prefill and decode throughput of the design (``--design``) and of its twin at each size, and the GPU time of a
     2,048-token prompt step and of a decode step at batch 8 by kernel class with each class's share of its
     roofline (weight bytes over 8 TB/s or flops over 2.5 PFLOP/s, whichever is longer). One JSON line."""
     import gc
@@ -469,8 +527,13 @@ def design_run(args) -> int:
         return out
 
     results = {}
-    for name, p_raw, q_raw, vocab in (kobolix_sizes() if args.design == "kobolix" else design_sizes()):
-        for which, raw in ((args.design, p_raw), ("qwen3", q_raw)):
+    sizes = {"kobolix": kobolix_sizes, "puresun": design_sizes, "detatar": detatar_sizes}[args.design]()
+    twin_name = "qwen3"
+    for name, p_raw, q_raw, vocab, *rest in sizes:
+        twin_name = rest[0] if rest else "qwen3"
+        if args.size and name != args.size:
+            continue
+        for which, raw in ((args.design, p_raw), (twin_name, q_raw)):
             cfg = config_from_dict(raw)
             log(f"{name} {which}: building ...")
             engine = LLMEngine(config=cfg, seed=args.seed, dtype=args.dtype, block_size=16,
@@ -498,7 +561,7 @@ def design_run(args) -> int:
             del engine
             gc.collect()
             torch.cuda.empty_cache()
-    print(json.dumps({"metric": f"{args.design}_beside_qwen3", "unit": "tokens/s", "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+    print(json.dumps({"metric": f"{args.design}_beside_{twin_name}", "unit": "tokens/s", "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
                       "data": "synthetic", "n_gpus": 1, "sizes": results}), flush=True)
     return 0
 
@@ -523,8 +586,10 @@ def main() -> int:
     ap.add_argument("--max-model-len", type=int, default=None, metavar="N",
                     help="context length (default: the shape's: 4096 at 8b, 8192 at 4b, 16384 at 32b)")
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes (default: the Qwen3-8B shape)")
-    ap.add_argument("--design", default=None, choices=["puresun", "kobolix"],
-                    help="instead of the default measurement: this design beside the Qwen3 decoder at equal sizes")
+    ap.add_argument("--design", default=None, choices=["puresun", "kobolix", "detatar"],
+                    help="instead of the default measurement: this design beside its closest other (the Qwen3 decoder; "
+                         "for detatar, Puresun) at equal sizes")
+    ap.add_argument("--size", default=None, help="with --design: this size alone (w2048 or w4096)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")

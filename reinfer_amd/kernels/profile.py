@@ -35,7 +35,9 @@ _OTHER = {"latent_prep": "latent norm + rotation + cache write", "head_linear": 
           "pair_hash_add": "embedding", "tanh_cap": "logit cap",
           "matrix_memory_scan": "matrix memory scan", "delta_rule_prepare": "filter + unit norms",
           "delta_rule_scan": "delta rule scan", "head_norm_gate": "head norm + gate",
-          "normed_mean": "mean of normed mixers", "moe_silu_gate_scale": "expert activation"}
+          "normed_mean": "mean of normed mixers", "moe_silu_gate_scale": "expert activation",
+          "wkv_scan": "wkv scan", "token_shift": "mix with the row before", "gated_stream_add": "gated stream add",
+          "rows_rmsnorm": "row norm", "tanh_rows": "tanh", "moe_identity_add": "identity experts"}
 
 
 class TimedKernels:

@@ -1,0 +1,136 @@
+"""Detatar configurations drawn at random (sizes, head counts, layer order, layers that run an earlier layer's
+tensors again, every optional section present or absent), each run through the engine against the plain
+implementation: a whole prompt, portions beside single tokens of other requests, and decoding, on a cache and state
+slots that are given back and taken again. In float32 as drawn; in bfloat16 with every router choosing all its
+experts (which of two nearly equal scores is the larger after rounding is decided differently by any two
+implementations)."""
+import json
+import os
+import random
+
+import pytest
+import torch
+
+import plain_detatar as plain
+from detatar_helpers import config_json, draw_weights, read_folder
+from helpers import random_tokens, rel_err, run_plan
+from test_detatar_engine import assert_close
+from reinfer_amd.engine import ModelRunner
+from reinfer_amd.weights.safetensors_io import write_safetensors
+
+pytestmark = pytest.mark.gpu
+
+
+def draw_config(rng: random.Random) -> dict:
+    groups = rng.choice([1, 1, 2, 3, 4])
+    width = groups * rng.choice([8, 12, 24, 40])
+
+    def wkv():
+        return {"dim": rng.choice([4, 9, 16, 32, 40, 64, 72]), "heads": rng.choice([1, 2, 3, 5])}
+
+    def latent():
+        rot_dim = rng.choice([2, 4, 8, 16, 32, 64])
+        m = {"dim": rng.choice([0, 8, 16, 24, 32, 64]), "heads": rng.choice([1, 2, 3, 4, 8, 16]),
+             "kv_rank": rng.choice([8, 24, 32, 64, 128]), "q_rank": rng.choice([4, 12, 48]), "rot_dim": rot_dim,
+             "scale": rng.choice([0.1, 0.25, 0.5]), "vdim": rng.choice([4, 8, 24, 32, 48]),
+             "rot": {"base": rng.choice([100.0, 10000.0, 1e6]), "dims": rot_dim}}
+        return m
+
+    def mlp():
+        kind = rng.choice(["dense", "moe", "moe", None])
+        if kind is None:
+            return None
+        if kind == "dense":
+            return {"ff": rng.choice([16, 40, 100]), "kind": "dense"}
+        count = rng.choice([1, 2, 3, 5])
+        per = rng.choice([1, 2, 4])
+        keep = rng.randint(1, count)
+        routed = count * per
+        identity = rng.choice([0, 0, 1, 2, 3])
+        identity = min(identity, routed - 1)
+        router = {"experts": routed - identity, "top": rng.randint(1, keep * per)}
+        if identity or rng.random() < 0.3:
+            router["identity"] = identity
+        if count > 1 or rng.random() < 0.5:
+            router["groups"] = {"count": count, "keep": keep}
+        out = {"expert": {"ff": rng.choice([8, 20, 48])}, "kind": "moe", "router": router}
+        if rng.random() < 0.6:
+            out["shared"] = {"ff": rng.choice([8, 36])}
+        return out
+
+    layers, ranks = [], []
+    for i in range(rng.randint(2, 5)):
+        own = [j for j, L in enumerate(layers) if "weights_of" not in L]
+        if own and rng.random() < 0.25:
+            j = rng.choice(own)
+            layers.append(dict(json.loads(json.dumps(layers[j])), weights_of=j))
+            ranks.append(0)
+            continue
+        if rng.random() < 0.45:
+            layers.append({"type": "wkv", "mixer": wkv(), "mlp": mlp()})
+            ranks.append(rng.choice([1, 4, 16, 24]))
+        else:
+            layers.append({"type": "latent_attention", "mixer": latent(), "mlp": mlp()})
+            ranks.append(0)
+    raw = {"architecture": "Detatar", "vocab": rng.choice([50, 131, 400]), "width": width,
+           "norm": {"eps": rng.choice([1e-6, 1e-5])}, "layers": layers, "decay_ranks": ranks}
+    if groups > 1 or rng.random() < 0.5:
+        raw["norm"]["groups"] = groups
+    if rng.random() < 0.8:
+        raw["embedding"] = {"scale": rng.choice([1.0, 3.0, 10.0])}
+    return raw
+
+
+@pytest.mark.parametrize("seed,dtype", [(s, "float32") for s in range(20)] + [(s, "bfloat16") for s in range(20, 30)])
+def test_random_configuration(tmp_path, seed, dtype):
+    rng = random.Random(2000 + seed)
+    raw = draw_config(rng)
+    if dtype == "bfloat16":
+        for L in raw["layers"]:
+            if L["mlp"] is not None and L["mlp"]["kind"] == "moe":
+                router = L["mlp"]["router"]
+                router["top"] = router["experts"] + router.get("identity", 0)
+                if "groups" in router:
+                    router["groups"]["keep"] = router["groups"]["count"]
+    print("configuration:", json.dumps(raw), flush=True)
+    folder = str(tmp_path / "m")
+    os.makedirs(folder)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(config_json(raw), f)
+    write_safetensors(os.path.join(folder, "model.safetensors"),
+                      draw_weights(raw, seed, torch.bfloat16 if dtype == "bfloat16" else torch.float32), metadata={"format": "pt"})
+    raw, w = read_folder(folder)
+    V = raw["vocab"]
+    lens = {"a": rng.randint(60, 140), "b": rng.randint(20, 70), "c": rng.randint(5, 40), "d": rng.randint(2, 30),
+            "e": rng.randint(30, 90)}
+    seqs = {r: random_tokens(n, V, seed * 10 + i) for i, (r, n) in enumerate(lens.items())}
+    refs = {r: plain.forward(raw, w, t).float() for r, t in seqs.items()}
+    # a plan of random portions: up to four live requests, the fifth comes when one has ended; the last tokens one by one
+    left = dict(lens)
+    waiting, live, plan = list(lens), [], []
+    while waiting or live:
+        while waiting and len(live) < 4:
+            live.append(waiting.pop(0))
+        items = []
+        for r in list(live):
+            if rng.random() < 0.25 and len(live) > 1:
+                continue                                            # left out of this step
+            c = 1 if left[r] <= 6 else min(left[r] - 6, rng.choice([1, 2, 3, 7, 16, 17, 33, 64]))
+            items.append((r, c))
+            left[r] -= c
+            if left[r] == 0:
+                live.remove(r)
+        if items:
+            plan.append(items)
+    runner = ModelRunner.from_folder(folder, dtype=dtype, device="cuda:0", max_tokens=4 * 192, max_seqs=4)
+    runner.poison_freed_blocks()
+    got = run_plan(runner, seqs, plan)
+    whole = run_plan(runner, {"a": seqs["a"]}, [[("a", lens["a"])]])["a"]
+    if dtype == "float32":
+        for r in seqs:
+            assert rel_err(got[r], refs[r]) < 3e-5, (r, json.dumps(raw))
+        assert rel_err(whole, refs["a"]) < 3e-5, json.dumps(raw)
+    else:
+        for r in seqs:
+            assert_close(got[r], refs[r], dtype, (r, json.dumps(raw)))
+        assert_close(whole, refs["a"], dtype, json.dumps(raw))
