@@ -28,6 +28,37 @@ template <> __device__ __forceinline__ float from_f32<float>(float v) { return v
 // round to nearest even; the hardware conversion of gfx950
 template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return (bf16_t)v; }
 
+// Eight consecutive elements as floats through 16-byte accesses; `p` is 16-byte aligned.
+template <typename T> struct Vec8;
+template <> struct Vec8<float> {
+  static __device__ __forceinline__ void load(const float* p, float (&v)[8]) {
+    const f32x4_t a = *(const f32x4_t*)p, b = *(const f32x4_t*)(p + 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { v[i] = a[i]; v[4 + i] = b[i]; }
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[8]) {
+    *(f32x4_t*)p = (f32x4_t){v[0], v[1], v[2], v[3]};
+    *(f32x4_t*)(p + 4) = (f32x4_t){v[4], v[5], v[6], v[7]};
+  }
+};
+template <> struct Vec8<bf16_t> {
+  static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[8]) {
+    const bf16x8_t a = *(const bf16x8_t*)p;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (float)a[i];
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[8]) {
+    bf16x8_t a;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) a[i] = (bf16_t)v[i];
+    *(bf16x8_t*)p = a;
+  }
+};
+// whether rows of `ld` elements of `bytes` each that start at `p` can be read in 16-byte pieces
+static inline bool ra_rows_16b(const void* p, long ld, int bytes) {
+  return p == nullptr || (((uintptr_t)p % 16) == 0 && (ld * bytes) % 16 == 0);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int m = RA_WAVE / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, RA_WAVE);

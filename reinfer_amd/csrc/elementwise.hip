@@ -224,15 +224,84 @@ __global__ void add_group_rmsnorm_kernel(float* __restrict__ resid, const TA* __
   }
 }
 
+// The same with a group's elements in registers: `wpg` waves share a group (their partial sums meet in shared
+// memory), each lane keeps at most GROUP_CH chunks of four. A decode step's few rows are then one read, one sum
+// and one write instead of two walks of the row by a single wave a group.
+#define GROUP_CH 4
+template <typename TA, typename TW>
+__global__ void add_group_rmsnorm_reg_kernel(float* __restrict__ resid, const TA* __restrict__ delta,
+                                             const TW* __restrict__ w, TA* __restrict__ out,
+                                             const int* __restrict__ rows, int h, int groups, int wpg, float eps,
+                                             float dscale) {
+  __shared__ float part[16];
+  const int r = blockIdx.x;
+  const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+  float* x = resid + src * h;
+  const TA* dl = delta ? delta + src * h : nullptr;
+  TA* o = out + (size_t)r * h;
+  const int lane = threadIdx.x & (RA_WAVE - 1);
+  const int wave = threadIdx.x / RA_WAVE, waves = blockDim.x / RA_WAVE;
+  const int gs = h / groups;
+  const int per_pass = waves / wpg;             // groups the workgroup takes at a time
+  const int sub = wave % wpg;
+  for (int g0 = 0; g0 < groups; g0 += per_pass) {    // every wave makes the same number of passes
+    const int g = g0 + wave / wpg;
+    const int base = g * gs;
+    f32x4_raw v[GROUP_CH];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < GROUP_CH; ++j) {
+      const int i = (lane + RA_WAVE * (sub + wpg * j)) * 4;
+      if (g < groups && i < gs) {
+        v[j] = Vec4<float>::load(x + base + i);
+        if (dl) {
+          v[j] += Vec4<TA>::load(dl + base + i) * dscale;
+          if (!rows) Vec4<float>::store(x + base + i, v[j]);
+        }
+        ss += v[j][0] * v[j][0] + v[j][1] * v[j][1] + v[j][2] * v[j][2] + v[j][3] * v[j][3];
+      }
+    }
+    ss = wave_sum(ss);
+    if (wpg > 1) {
+      __syncthreads();                          // the pass before has read its sums
+      if (lane == 0) part[wave] = ss;
+      __syncthreads();
+      ss = 0.f;
+      const int w0 = wave - sub;
+      for (int k = 0; k < wpg; ++k) ss += part[w0 + k];     // the same order in every wave of the group
+    }
+    const float rstd = rsqrtf(ss / (float)gs + eps);
+#pragma unroll
+    for (int j = 0; j < GROUP_CH; ++j) {
+      const int i = (lane + RA_WAVE * (sub + wpg * j)) * 4;
+      if (g < groups && i < gs) Vec4<TA>::store(o + base + i, v[j] * rstd * Vec4<TW>::load(w + base + i));
+    }
+  }
+}
+
 extern "C" int ra_add_group_rmsnorm(float* resid, const void* delta, const void* weight, int weight_dtype,
                                     void* out, int act_dtype, const int* rows, int n_rows, int hidden, int groups,
                                     float eps, float delta_scale, hipStream_t stream) {
   RA_CHECK(n_rows > 0 && hidden > 0, "add_group_rmsnorm: empty input (%d rows, width %d)", n_rows, hidden);
   RA_CHECK(groups >= 1 && hidden % groups == 0, "add_group_rmsnorm: width %d in %d equal groups", hidden, groups);
   const int threads = RA_WAVE * (groups >= 8 ? 8 : groups >= 4 ? 4 : groups >= 2 ? 2 : 1);
-#define RA_GN(TA, TW)                                                                                          \
-  add_group_rmsnorm_kernel<TA, TW><<<n_rows, threads, 0, stream>>>(resid, (const TA*)delta, (const TW*)weight, \
-                                                                   (TA*)out, rows, hidden, groups, eps, delta_scale)
+  const int gs = hidden / groups;
+  // waves a group: as many as a group of this size can feed with one chunk a lane, within eight waves a workgroup
+  int wpg = 1;
+  while (wpg * 2 * groups <= 8 && gs >= wpg * 2 * RA_WAVE * 4) wpg *= 2;
+  const int reg_waves = groups >= 8 ? 8 : groups * wpg;
+  const bool in_regs = gs % 4 == 0 && gs <= wpg * RA_WAVE * 4 * GROUP_CH && ((uintptr_t)resid % 16) == 0 &&
+                       ((uintptr_t)out % 16) == 0 && ((uintptr_t)weight % 16) == 0 && ((uintptr_t)delta % 16) == 0;
+#define RA_GN(TA, TW)                                                                                                \
+  do {                                                                                                               \
+    if (in_regs)                                                                                                     \
+      add_group_rmsnorm_reg_kernel<TA, TW><<<n_rows, reg_waves * RA_WAVE, 0, stream>>>(                              \
+          resid, (const TA*)delta, (const TW*)weight, (TA*)out, rows, hidden, groups, wpg, eps, delta_scale);        \
+    else                                                                                                             \
+      add_group_rmsnorm_kernel<TA, TW><<<n_rows, threads, 0, stream>>>(resid, (const TA*)delta, (const TW*)weight,   \
+                                                                       (TA*)out, rows, hidden, groups, eps,          \
+                                                                       delta_scale);                                 \
+  } while (0)
   if (act_dtype == RA_F32 && weight_dtype == RA_F32) RA_GN(float, float);
   else if (act_dtype == RA_BF16 && weight_dtype == RA_BF16) RA_GN(bf16_t, bf16_t);
   else if (act_dtype == RA_BF16 && weight_dtype == RA_F32) RA_GN(bf16_t, float);
@@ -835,7 +904,8 @@ extern "C" int ra_qk_norm_rope_cache_sums(const float* parts, int n_ranges, cons
 // ---------------------------------------------------------------------------
 // act 0: silu; act 1: the tanh form of gelu, 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
 __device__ __forceinline__ float gate_act(float g, int act) {
-  if (act == 1) return 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+  // 0.5 (1 + tanh y) = 1 / (1 + exp(-2 y))
+  if (act == 1) return g / (1.f + expf(-1.5957691216057308f * (g + 0.044715f * g * g * g)));
   return g / (1.f + expf(-g));
 }
 

@@ -92,15 +92,17 @@ def test_wkv_bonus_decay_and_order_by_hand():
     close(out, want, 1e-6, "by hand")
 
 
-@pytest.mark.parametrize("width,n_mix", [(64, 1), (36, 5), (200, 5), (1024, 1), (8, 2)])
+@pytest.mark.parametrize("width,n_mix,tail", [(64, 1, 2), (36, 5, 2), (200, 5, 2), (1024, 1, 2), (8, 2, 2), (64, 2, 8), (200, 5, 0),
+                                              (4096, 5, 4), (1032, 3, 0), (2048, 1, 2)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_token_shift(width, n_mix, dtype):
+def test_token_shift(width, n_mix, tail, dtype):
     ops, ref = kernels.current(), KernelDouble()
     g = torch.Generator().manual_seed(width + n_mix)
     mu = torch.rand(n_mix, width, generator=g).to(dtype)
     keep_off = 24
-    st_gpu = torch.full((4, keep_off + width + 2), float("nan"), device=DEV)
-    st_ref = torch.full((4, keep_off + width + 2), float("nan"))
+    # a state row of a whole number of 16 bytes (tail a multiple of 4 here) is read 16 bytes a thread
+    st_gpu = torch.full((4, keep_off + width + tail), float("nan"), device=DEV)
+    st_ref = torch.full((4, keep_off + width + tail), float("nan"))
     for i, (q_lens, slots, fresh) in enumerate(CALLS):
         T = sum(q_lens)
         wide = torch.randn(T, width + 8, generator=g).to(dtype)
@@ -114,7 +116,7 @@ def test_token_shift(width, n_mix, dtype):
         assert torch.isnan(st_gpu[:, :keep_off]).all() and torch.isnan(st_gpu[:, keep_off + width:]).all()
 
 
-@pytest.mark.parametrize("width", [36, 64, 1000])
+@pytest.mark.parametrize("width", [36, 64, 1000, 4096, 520])
 @pytest.mark.parametrize("both", [True, False])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_gated_stream_add(width, both, dtype):
@@ -132,7 +134,8 @@ def test_gated_stream_add(width, both, dtype):
     close(got, want, 1e-6, "stream")
 
 
-@pytest.mark.parametrize("width,groups", [(64, 4), (36, 3), (192, 1), (1000, 8), (40, 5)])
+@pytest.mark.parametrize("width,groups", [(64, 4), (36, 3), (192, 1), (1000, 8), (40, 5), (4096, 4), (2048, 1), (1536, 3),
+                                          (8192, 2), (16384, 2), (2560, 10), (1792, 7)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_norm_in_groups(width, groups, dtype):
     ops, ref = kernels.current(), KernelDouble()
@@ -164,7 +167,7 @@ def test_rows_norm_tanh_and_gelu(dtype):
     ops, ref = kernels.current(), KernelDouble()
     g = torch.Generator().manual_seed(8)
     T = 21
-    for width in (24, 80, 1536):
+    for width in (24, 80, 1536, 2048, 2056):
         wide = (torch.randn(T, width + 16, generator=g) * 3).to(dtype)
         weight = (torch.rand(width, generator=g) + 0.5).to(dtype)
         out_ref, out = torch.empty(T, width, dtype=dtype), torch.empty(T, width, dtype=dtype, device=DEV)
