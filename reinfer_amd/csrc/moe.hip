@@ -348,6 +348,49 @@ __global__ void moe_silu_gate_scale_kernel(const TA* __restrict__ gu, TA* __rest
   act[(size_t)t * n + i] = from_f32<TA>(p * (g / (1.f + expf(-g))) * u);
 }
 
+// the same, eight columns a thread through 16-byte accesses (ff and shared multiples of 8: the eight lie in one
+// expert, or in the shared one)
+template <typename TA>
+__global__ void moe_silu_gate_scale_x8_kernel(const TA* __restrict__ gu, TA* __restrict__ act,
+                                              const int* __restrict__ ids, const float* __restrict__ weights, int top,
+                                              int E, int ff, int shared, const float* __restrict__ shared_logit,
+                                              int ld_logit) {
+  extern __shared__ float gate[];        // [E]
+  const int t = blockIdx.y;
+  for (int e = threadIdx.x; e < E; e += blockDim.x) gate[e] = 0.f;
+  __syncthreads();
+  for (int j = threadIdx.x; j < top; j += blockDim.x) {
+    const int id = ids[(size_t)t * top + j];
+    if (id < E) gate[id] = weights[(size_t)t * top + j];
+  }
+  __syncthreads();
+  const int n = E * ff + shared;
+  const int i = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  if (i >= n) return;
+  const TA* row = gu + (size_t)t * 2 * n;
+  float p, g[8], u[8];
+  if (i < E * ff) {
+    const int e = i / ff, j = i - e * ff;
+    p = gate[e];
+    if (p == 0.f) {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) g[k] = 0.f;
+      Vec8<TA>::store(act + (size_t)t * n + i, g);
+      return;
+    }
+    Vec8<TA>::load(row + (size_t)e * 2 * ff + j, g);
+    Vec8<TA>::load(row + (size_t)e * 2 * ff + ff + j, u);
+  } else {
+    const int j = i - E * ff;
+    p = shared_logit ? 1.f / (1.f + expf(-shared_logit[(size_t)t * ld_logit])) : 1.f;
+    Vec8<TA>::load(row + (size_t)E * 2 * ff + j, g);
+    Vec8<TA>::load(row + (size_t)E * 2 * ff + shared + j, u);
+  }
+#pragma unroll
+  for (int k = 0; k < 8; ++k) g[k] = p * (g[k] / (1.f + expf(-g[k]))) * u[k];
+  Vec8<TA>::store(act + (size_t)t * n + i, g);
+}
+
 extern "C" int ra_moe_silu_gate_scale(const void* gu, void* act, int act_dtype, const int* ids, const float* weights,
                                       int top, int experts, int ff, int shared, int n_tokens, hipStream_t stream) {
   return ra_moe_silu_gate_scale_shared(gu, act, act_dtype, ids, weights, top, experts, ff, shared, nullptr, 0, n_tokens,
@@ -365,6 +408,18 @@ extern "C" int ra_moe_silu_gate_scale_shared(const void* gu, void* act, int act_
   RA_CHECK(lds <= 64 * 1024, "moe_silu_gate_scale: %d experts", experts);
   const int n = experts * ff + shared;
   dim3 grid((n + 255) / 256, n_tokens);
+  if (ff % 8 == 0 && shared % 8 == 0 && ((uintptr_t)gu % 16) == 0 && ((uintptr_t)act % 16) == 0 &&
+      (act_dtype == RA_F32 || act_dtype == RA_BF16)) {
+    dim3 grid8((n / 8 + 255) / 256, n_tokens);
+    if (act_dtype == RA_F32)
+      moe_silu_gate_scale_x8_kernel<float><<<grid8, 256, lds, stream>>>((const float*)gu, (float*)act, ids, weights, top,
+                                                                        experts, ff, shared, shared_logit, ld_logit);
+    else
+      moe_silu_gate_scale_x8_kernel<bf16_t><<<grid8, 256, lds, stream>>>((const bf16_t*)gu, (bf16_t*)act, ids, weights,
+                                                                         top, experts, ff, shared, shared_logit, ld_logit);
+    RA_LAUNCH_CHECK("moe_silu_gate_scale");
+    return 0;
+  }
   if (act_dtype == RA_F32)
     moe_silu_gate_scale_kernel<float><<<grid, 256, lds, stream>>>((const float*)gu, (float*)act, ids, weights, top,
                                                                    experts, ff, shared, shared_logit, ld_logit);
@@ -585,5 +640,146 @@ extern "C" int ra_moe_down_chosen(const void* act, const void* w_down, const int
   else
     return ra_fail("moe_down_chosen: unknown dtype tag %d", act_dtype);
   RA_LAUNCH_CHECK("moe_down_chosen");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// The same for gated experts whose [gate; up] rows lie one expert after the other in one matrix, a shared
+// expert's behind them, and whose down projections lie side by side, the shared one's last. Pair p = (token t,
+// choice j), j < top; with a shared expert one more pair a token, j = top. act is [T, top * ff + shared]:
+//   act[t, j * ff + f]   = g * silu(W[e 2 ff + f, :] . x[t]) * (W[e 2 ff + ff + f, :] . x[t])     e = ids[t, j], g = weights[t, j]
+//   act[t, top * ff + f] = g_s * silu(W[E 2 ff + f, :] . x[t]) * (W[E 2 ff + shared + f, :] . x[t])
+//                          g_s = sigmoid(shared_logit[t]) or 1
+//   y[t, n] = sum_j Wd[n, e_j ff : (e_j + 1) ff] . act[t, j ff : ...] + Wd[n, E ff :] . act[t, top ff :]
+//             + (sum of g over choices with e >= E) * x[t, n]
+// A chosen id of E or more names no matrices (an identity expert): its part of act is zero and not read.
+// ---------------------------------------------------------------------------
+template <typename TA>
+__global__ void __launch_bounds__(256)
+moe_gate_up_chosen_kernel(const TA* __restrict__ x, int ldx, const TA* __restrict__ Wgu, const int* __restrict__ ids,
+                          const float* __restrict__ weights, const float* __restrict__ shared_logit, int ld_logit,
+                          TA* __restrict__ act, int ff, int shared, int E, int width, int top, int vec) {
+  const int lane = threadIdx.x & (RA_WAVE - 1);
+  const int wave = threadIdx.x / RA_WAVE;
+  const int per_token = top + (shared > 0 ? 1 : 0);
+  const int t = blockIdx.y / per_token, j = blockIdx.y - t * per_token;
+  const bool is_shared = j == top;
+  const int rows = is_shared ? shared : ff;
+  const int f0 = blockIdx.x * MOE_ROWS + wave * 4;
+  if (f0 >= rows) return;
+  TA* o = act + (size_t)t * ((size_t)top * ff + shared) + (size_t)j * ff;
+  const int e = is_shared ? E : ids[t * top + j];
+  if (e > E || (e == E && !is_shared)) {          // an identity expert
+    if (lane < 4 && f0 + lane < rows) o[f0 + lane] = from_f32<TA>(0.f);
+    return;
+  }
+  const float g = is_shared ? (shared_logit ? 1.f / (1.f + expf(-shared_logit[(size_t)t * ld_logit])) : 1.f)
+                            : weights[t * top + j];
+  const TA* base = Wgu + (size_t)e * 2 * ff * width;          // the shared expert's rows lie behind E experts'
+  const TA* wg[4];
+  const TA* wu[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int f = f0 + r < rows ? f0 + r : f0;                 // past the end: a row again, not stored
+    wg[r] = base + (size_t)f * width;
+    wu[r] = base + (size_t)(rows + f) * width;
+  }
+  float sg[4] = {0.f, 0.f, 0.f, 0.f}, su[4] = {0.f, 0.f, 0.f, 0.f};
+  moe_dot4<TA>(wg, x + (size_t)t * ldx, width, lane, vec != 0, sg);
+  moe_dot4<TA>(wu, x + (size_t)t * ldx, width, lane, vec != 0, su);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    sg[r] = wave_sum(sg[r]);
+    su[r] = wave_sum(su[r]);
+  }
+  if (lane < 4 && f0 + lane < rows) {
+    const float a = lane == 0 ? sg[0] : lane == 1 ? sg[1] : lane == 2 ? sg[2] : sg[3];
+    const float u = lane == 0 ? su[0] : lane == 1 ? su[1] : lane == 2 ? su[2] : su[3];
+    o[f0 + lane] = from_f32<TA>(g * (a / (1.f + expf(-a))) * u);
+  }
+}
+
+template <typename TA>
+__global__ void __launch_bounds__(256)
+moe_down_gated_chosen_kernel(const TA* __restrict__ act, const TA* __restrict__ Wdown, const int* __restrict__ ids,
+                             const float* __restrict__ weights, const TA* __restrict__ x, int ldx,
+                             TA* __restrict__ out, int ff, int shared, int width, int E, int top, int vec) {
+  const int lane = threadIdx.x & (RA_WAVE - 1);
+  const int wave = threadIdx.x / RA_WAVE;
+  const int t = blockIdx.y;
+  const int n0 = blockIdx.x * MOE_ROWS + wave * 4;
+  if (n0 >= width) return;
+  const size_t ldw = (size_t)E * ff + shared, lda = (size_t)top * ff + shared;
+  float s[4] = {0.f, 0.f, 0.f, 0.f};
+  float coef = 0.f;
+  const TA* w[4];
+  for (int j = 0; j < top; ++j) {               // choice order: the same sum whatever else is in the step
+    const int e = ids[t * top + j];
+    if (e >= E) {
+      coef += weights[t * top + j];
+      continue;
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) w[r] = Wdown + (size_t)(n0 + r < width ? n0 + r : n0) * ldw + (size_t)e * ff;
+    moe_dot4<TA>(w, act + t * lda + (size_t)j * ff, ff, lane, vec != 0, s);
+  }
+  if (shared > 0) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) w[r] = Wdown + (size_t)(n0 + r < width ? n0 + r : n0) * ldw + (size_t)E * ff;
+    moe_dot4<TA>(w, act + t * lda + (size_t)top * ff, shared, lane, vec != 0, s);
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) s[r] = wave_sum(s[r]);
+  if (lane < 4 && n0 + lane < width) {
+    float v = lane == 0 ? s[0] : lane == 1 ? s[1] : lane == 2 ? s[2] : s[3];
+    if (coef != 0.f) v += coef * to_f32(x[(size_t)t * ldx + n0 + lane]);
+    out[(size_t)t * width + n0 + lane] = from_f32<TA>(v);
+  }
+}
+
+extern "C" int ra_moe_gate_up_chosen(const void* x, int ldx, const void* w_gate_up, const int* ids, const float* weights,
+                                     const float* shared_logit, int ld_logit, void* act, int act_dtype, int n_tokens,
+                                     int top, int experts, int ff, int shared, int width, hipStream_t stream) {
+  RA_CHECK(n_tokens > 0 && top > 0 && experts > 0 && ff > 0 && shared >= 0 && width > 0 && ldx >= width,
+           "moe_gate_up_chosen: %d tokens, %d of %d experts of %d x %d, shared %d", n_tokens, top, experts, ff, width, shared);
+  const long pairs = (long)n_tokens * (top + (shared > 0 ? 1 : 0));
+  RA_CHECK(pairs <= 65535, "moe_gate_up_chosen: %ld pairs in one launch", pairs);
+  const int vec = (width % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w_gate_up % 16) == 0) ? 1 : 0;
+  const int rows = ff > shared ? ff : shared;
+  dim3 grid((rows + MOE_ROWS - 1) / MOE_ROWS, (unsigned)pairs);
+  if (act_dtype == RA_F32)
+    moe_gate_up_chosen_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, ldx, (const float*)w_gate_up, ids, weights,
+                                                               shared_logit, ld_logit, (float*)act, ff, shared, experts,
+                                                               width, top, 0);
+  else if (act_dtype == RA_BF16)
+    moe_gate_up_chosen_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w_gate_up, ids,
+                                                                weights, shared_logit, ld_logit, (bf16_t*)act, ff, shared,
+                                                                experts, width, top, vec);
+  else
+    return ra_fail("moe_gate_up_chosen: unknown dtype tag %d", act_dtype);
+  RA_LAUNCH_CHECK("moe_gate_up_chosen");
+  return 0;
+}
+
+extern "C" int ra_moe_down_gated_chosen(const void* act, const void* w_down, const int* ids, const float* weights,
+                                        const void* x, int ldx, void* out, int act_dtype, int n_tokens, int top,
+                                        int experts, int ff, int shared, int width, hipStream_t stream) {
+  RA_CHECK(n_tokens > 0 && top > 0 && experts > 0 && ff > 0 && shared >= 0 && width > 0 && ldx >= width,
+           "moe_down_gated_chosen: %d tokens, %d of %d experts of %d x %d, shared %d", n_tokens, top, experts, ff, width, shared);
+  RA_CHECK(n_tokens <= 65535, "moe_down_gated_chosen: %d tokens in one launch", n_tokens);
+  RA_CHECK(act != nullptr && out != nullptr && x != nullptr, "moe_down_gated_chosen: act, x and out are given");
+  const int vec = (ff % 8 == 0 && shared % 8 == 0 && ((uintptr_t)act % 16) == 0 && ((uintptr_t)w_down % 16) == 0) ? 1 : 0;
+  dim3 grid((width + MOE_ROWS - 1) / MOE_ROWS, n_tokens);
+  if (act_dtype == RA_F32)
+    moe_down_gated_chosen_kernel<float><<<grid, 256, 0, stream>>>((const float*)act, (const float*)w_down, ids, weights,
+                                                                  (const float*)x, ldx, (float*)out, ff, shared, width,
+                                                                  experts, top, 0);
+  else if (act_dtype == RA_BF16)
+    moe_down_gated_chosen_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)w_down, ids, weights,
+                                                                   (const bf16_t*)x, ldx, (bf16_t*)out, ff, shared, width,
+                                                                   experts, top, vec);
+  else
+    return ra_fail("moe_down_gated_chosen: unknown dtype tag %d", act_dtype);
+  RA_LAUNCH_CHECK("moe_down_gated_chosen");
   return 0;
 }

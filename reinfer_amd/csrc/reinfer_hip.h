@@ -5,7 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define RA_ABI_VERSION 21
+#define RA_ABI_VERSION 22
 
 #ifdef __cplusplus
 extern "C" {
@@ -245,6 +245,19 @@ int ra_moe_route_softmax(const float* logits, int ld, int experts, int top, int 
 // identity
 int ra_moe_identity_add(void* y, int ldy, const void* x, int ldx, int act_dtype, const int* ids, const float* weights,
                         int top, int experts, int n_tokens, int width, hipStream_t stream);
+
+// Few tokens, gated experts: only the chosen experts' rows are read, and the shared expert's. w_gate_up
+// [2 (experts ff + shared), width], [gate; up] an expert, the shared expert's last; w_down [width, experts ff + shared].
+// act [n_tokens, top ff + shared]: act[t, j ff + f] = weights[t, j] silu(gate) up of expert ids[t, j] (0 for an id of
+// `experts` or more), behind them the shared expert's, times sigmoid(shared_logit[t * ld_logit]) (null: 1). Then
+// out[t, n] = sum_j w_down[n, ids[t, j] ff : ...] . act[t, j ff : ...] + w_down[n, experts ff :] . act[t, top ff :]
+//             + (sum of weights[t, j] with ids[t, j] >= experts) * x[t, n]
+int ra_moe_gate_up_chosen(const void* x, int ldx, const void* w_gate_up, const int* ids, const float* weights,
+                          const float* shared_logit, int ld_logit, void* act, int act_dtype, int n_tokens, int top,
+                          int experts, int ff, int shared, int width, hipStream_t stream);
+int ra_moe_down_gated_chosen(const void* act, const void* w_down, const int* ids, const float* weights, const void* x,
+                             int ldx, void* out, int act_dtype, int n_tokens, int top, int experts, int ff, int shared,
+                             int width, hipStream_t stream);
 
 // C += acc_scale * (A . W^T) through the weight-streaming kernels (bfloat16 operands, float C; the limits of
 // ra_gemm_skinny / ra_gemm_wide with the accumulating epilogue)

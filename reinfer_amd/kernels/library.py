@@ -15,7 +15,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library links against)
 
 from ..csrc import build as _build
 
-ABI_VERSION = 21
+ABI_VERSION = 22
 
 
 class KernelLibraryError(RuntimeError):
@@ -68,6 +68,8 @@ _SIGNATURES = {
     "ra_moe_relu2_scale": [P, P, I, P, P, I, I, I, I, P],
     "ra_moe_up_chosen": [P, I, P, P, P, P, I, I, I, I, I, I, P],
     "ra_moe_down_chosen": [P, P, P, P, P, I, I, I, I, I, I, P],
+    "ra_moe_gate_up_chosen": [P, I, P, P, P, P, I, P, I, I, I, I, I, I, I, P],
+    "ra_moe_down_gated_chosen": [P, P, P, P, P, I, P, I, I, I, I, I, I, I, P],
     "ra_moe_route_sigmoid": [P, I, I, I, I, I, I, F, P, P, I, P],
     "ra_moe_silu_gate_scale": [P, P, I, P, P, I, I, I, I, I, P],
     "ra_matrix_memory_scan": [P, I, I, I, I, I, P, P, P, P, c_long, P, P, P, I, I, I, I, I, I, F, F, F, P, P],

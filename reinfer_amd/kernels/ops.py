@@ -1381,6 +1381,54 @@ class HipKernels:
         library.call("ra_moe_down_chosen", act.data_ptr(), w_down.data_ptr(), ids.data_ptr(), _ptr(resid), _ptr(out),
                      _tag(act, "moe_down_chosen"), T, top, E, int(ff), width, _stream())
 
+    def moe_gate_up_chosen(self, x: torch.Tensor, w_gate_up: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor,
+                           act: torch.Tensor, experts: int, ff: int, shared: int,
+                           shared_logit: Optional[torch.Tensor] = None) -> None:
+        """Gated experts, the chosen ones only: act[t, j * ff : ...] = weights[t, j] * silu(W_gate x[t]) * (W_up x[t])
+        of expert ids[t, j] (zeros for an id of ``experts`` or more), and behind the ``top`` choices the shared
+        expert's, times sigmoid(shared_logit[t]) where that is given. ``w_gate_up`` is [2 (experts ff + shared),
+        width] with [gate; up] an expert, the shared expert's last; ``act`` [T, top * ff + shared]."""
+        _dev(x, w_gate_up, ids, weights, act)
+        T, width = x.shape
+        top = ids.shape[1]
+        if w_gate_up.shape != (2 * (experts * ff + shared), width) or not w_gate_up.is_contiguous() \
+                or x.dtype != w_gate_up.dtype or x.stride(1) != 1:
+            raise ValueError(f"moe_gate_up_chosen: x {tuple(x.shape)}, w_gate_up {tuple(w_gate_up.shape)} for "
+                             f"{experts} experts of {ff} and a shared one of {shared}")
+        if act.shape != (T, top * ff + shared) or act.dtype != x.dtype or not act.is_contiguous():
+            raise ValueError(f"moe_gate_up_chosen: act {tuple(act.shape)}, expected [{T}, {top * ff + shared}]")
+        self._check_choice("moe_gate_up_chosen", ids, weights, T, top)
+        ld = 0
+        if shared_logit is not None:
+            _dev(shared_logit)
+            if shared_logit.dtype != torch.float32 or shared_logit.shape[0] != T or shared_logit.numel() != T:
+                raise ValueError("moe_gate_up_chosen: the shared expert's logits are float32, one a token")
+            ld = shared_logit.stride(0)
+        library.call("ra_moe_gate_up_chosen", x.data_ptr(), x.stride(0), w_gate_up.data_ptr(), ids.data_ptr(),
+                     weights.data_ptr(), _ptr(shared_logit), int(ld), act.data_ptr(), _tag(x, "moe_gate_up_chosen"), T,
+                     top, int(experts), int(ff), int(shared), width, _stream())
+
+    def moe_down_gated_chosen(self, act: torch.Tensor, w_down: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor,
+                              x: torch.Tensor, out: torch.Tensor, experts: int, ff: int, shared: int) -> None:
+        """out[t] = sum_j w_down[:, ids[t, j] * ff : ...] . act[t, j * ff : ...] + the shared expert's columns times
+        its part of act + (the weights of chosen ids of ``experts`` or more) * x[t]; ``w_down`` is
+        [width, experts * ff + shared], ``act`` as ``moe_gate_up_chosen`` leaves it."""
+        _dev(act, w_down, ids, weights, x, out)
+        T, top = ids.shape
+        width = w_down.shape[0]
+        if w_down.shape != (width, experts * ff + shared) or not w_down.is_contiguous() or act.dtype != w_down.dtype \
+                or act.shape != (T, top * ff + shared) or not act.is_contiguous():
+            raise ValueError(f"moe_down_gated_chosen: act {tuple(act.shape)}, w_down {tuple(w_down.shape)} for "
+                             f"{experts} experts of {ff} and a shared one of {shared}")
+        self._check_choice("moe_down_gated_chosen", ids, weights, T, top)
+        if x.shape != (T, width) or x.dtype != act.dtype or x.stride(1) != 1:
+            raise ValueError(f"moe_down_gated_chosen: x {tuple(x.shape)}, expected [{T}, {width}]")
+        if out.shape != (T, width) or out.dtype != act.dtype or not out.is_contiguous():
+            raise ValueError("moe_down_gated_chosen: out is contiguous [T, width] in the activations' dtype")
+        library.call("ra_moe_down_gated_chosen", act.data_ptr(), w_down.data_ptr(), ids.data_ptr(), weights.data_ptr(),
+                     x.data_ptr(), x.stride(0), out.data_ptr(), _tag(act, "moe_down_gated_chosen"), T, top,
+                     int(experts), int(ff), int(shared), width, _stream())
+
     @staticmethod
     def _check_choice(what: str, ids, weights, T: int, top: int) -> None:
         if ids.shape != (T, top) or ids.dtype != torch.int32 or not ids.is_contiguous() \

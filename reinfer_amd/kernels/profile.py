@@ -31,7 +31,8 @@ _LINEAR = {"linear", "linear_plain", "linear_skinny", "gated_linear", "linear_ra
 # kernels of further mechanisms, each a class of its own
 _OTHER = {"latent_prep": "latent norm + rotation + cache write", "head_linear": "products head by head",
           "moe_route": "router", "moe_relu2_scale": "expert activation",
-          "moe_up_chosen": "chosen experts up", "moe_down_chosen": "chosen experts down", "stream_add": "stream add",
+          "moe_up_chosen": "chosen experts up", "moe_down_chosen": "chosen experts down",
+          "moe_gate_up_chosen": "chosen experts up", "moe_down_gated_chosen": "chosen experts down", "stream_add": "stream add",
           "pair_hash_add": "embedding", "tanh_cap": "logit cap",
           "matrix_memory_scan": "matrix memory scan", "delta_rule_prepare": "filter + unit norms",
           "delta_rule_scan": "delta rule scan", "head_norm_gate": "head norm + gate",

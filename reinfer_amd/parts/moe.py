@@ -19,7 +19,8 @@ best groups can be chosen; the chosen experts' weights are their scores times a 
 a shared expert of the same form may run for every token. Here every expert's [gate; up] rows lie one
 after the other in one matrix, the shared expert's behind them, one kernel applies the gate and the
 routing weight (1 for the shared expert, 0 for experts not chosen), and one product with all down
-projections side by side is the sum.
+projections side by side is the sum. A step of few tokens reads only the chosen experts' rows and the shared
+expert's, as the first form does.
 
 A third form (``activation`` "silu_gated", ``weights`` "softmax"): scores are the softmax of the router's logits
 over all its outputs; the choice is by score + a stored correction, inside the best groups (a group's score is
@@ -134,6 +135,16 @@ class MixtureOfExperts:
         else:
             ops.moe_route(x, self.router, self.top, ids, weights, scoring="sigmoid", scale=float(p.weight_scale),
                           groups=int(p.groups), groups_kept=int(p.groups_kept), group_top=int(p.group_top))
+        chosen = getattr(ops, "moe_reads_chosen", None)
+        if chosen is not None and hasattr(ops, "moe_gate_up_chosen") and chosen(T, self.top, routed):
+            # so few tokens that most experts are not asked for: only the chosen experts' rows and the shared
+            # expert's are read; the identity experts' share is added behind the down projection's sum
+            act = torch.empty((T, self.top * self.ff + self.shared), dtype=self.dtype, device=x.device)
+            ops.moe_gate_up_chosen(x, self.w_gate_up, ids, weights, act, self.experts, self.ff, self.shared,
+                                   shared_logit=shared_logit)
+            out = torch.empty((T, self.spec.hidden), dtype=self.dtype, device=x.device)
+            ops.moe_down_gated_chosen(act, self.w_down, ids, weights, x, out, self.experts, self.ff, self.shared)
+            return out
         gu = torch.empty((T, 2 * n), dtype=self.dtype, device=x.device)
         ops.linear(x, self.w_gate_up, gu)
         act = torch.empty((T, n), dtype=self.dtype, device=x.device)

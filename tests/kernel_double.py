@@ -392,6 +392,39 @@ class KernelDouble:
             else:
                 out[t] = y.to(out.dtype)
 
+    def moe_gate_up_chosen(self, x, w_gate_up, ids, weights, act, experts, ff, shared, shared_logit=None):
+        T, top = ids.shape
+        act.zero_()
+        for t in range(T):
+            xt = x[t].float()
+            for j in range(top):
+                e = int(ids[t, j])
+                if e >= experts:
+                    continue
+                g = w_gate_up[e * 2 * ff:e * 2 * ff + ff].float() @ xt
+                u = w_gate_up[e * 2 * ff + ff:(e + 1) * 2 * ff].float() @ xt
+                act[t, j * ff:(j + 1) * ff] = (float(weights[t, j]) * g * torch.sigmoid(g) * u).to(act.dtype)
+            if shared:
+                b = experts * 2 * ff
+                g = w_gate_up[b:b + shared].float() @ xt
+                u = w_gate_up[b + shared:].float() @ xt
+                sw = torch.sigmoid(shared_logit[t].float()) if shared_logit is not None else 1.0
+                act[t, top * ff:] = (sw * g * torch.sigmoid(g) * u).to(act.dtype)
+
+    def moe_down_gated_chosen(self, act, w_down, ids, weights, x, out, experts, ff, shared):
+        T, top = ids.shape
+        for t in range(T):
+            y = torch.zeros(w_down.shape[0])
+            for j in range(top):
+                e = int(ids[t, j])
+                if e >= experts:
+                    y += float(weights[t, j]) * x[t].float()
+                else:
+                    y += w_down[:, e * ff:(e + 1) * ff].float() @ act[t, j * ff:(j + 1) * ff].float()
+            if shared:
+                y += w_down[:, experts * ff:].float() @ act[t, top * ff:].float()
+            out[t] = y.to(out.dtype)
+
     GATE_GROUP = 8
 
     def silu_mul(self, gate_up, out, group=0, act="silu"):

@@ -238,7 +238,8 @@ def test_moe_route_softmax_by_hand():
     assert torch.allclose(w, torch.tensor([0.5, 0.5]), atol=1e-6)
 
 
-@pytest.mark.parametrize("E,ident,ff,shared,top", [(6, 2, 24, 40, 3), (3, 1, 7, 0, 4), (4, 0, 10, 3, 2), (2, 3, 16, 8, 5)])
+@pytest.mark.parametrize("E,ident,ff,shared,top", [(6, 2, 24, 40, 3), (3, 1, 7, 0, 4), (4, 0, 10, 3, 2), (2, 3, 16, 8, 5),
+                                                   (14, 2, 1024, 2048, 4)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_identity_experts_and_the_shared_experts_sigmoid(E, ident, ff, shared, top, dtype):
     ops, ref = kernels.current(), KernelDouble()
@@ -261,6 +262,50 @@ def test_identity_experts_and_the_shared_experts_sigmoid(E, ident, ff, shared, t
     ref.moe_identity_add(y_ref, x, ids, w, E)
     ops.moe_identity_add(y_gpu, x.to(DEV), ids.to(DEV), w.to(DEV), E)
     close(y_gpu, y_ref, 1e-6 if dtype == torch.float32 else 1e-2, "identity")
+
+
+@pytest.mark.parametrize("E,ident,ff,shared,top,width", [(6, 2, 24, 40, 3, 64), (3, 1, 7, 0, 4, 40), (4, 0, 10, 3, 2, 36),
+                                                         (2, 3, 16, 8, 5, 128), (14, 2, 64, 128, 4, 512), (5, 1, 32, 8, 2, 72)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gated_experts_read_chosen_only(E, ident, ff, shared, top, width, dtype):
+    """The few-token path against the plain double, and against the path that runs every expert: the same
+    function of the same choices, the identity experts' share and the shared expert's sigmoid included."""
+    ops, ref = kernels.current(), KernelDouble()
+    g = torch.Generator().manual_seed(ff + ident + width)
+    T = 5
+    n = E * ff + shared
+    x = torch.randn(T, width + 8, generator=g).to(dtype)[:, 8:]
+    w_gu = (torch.randn(2 * n, width, generator=g) * width ** -0.5).to(dtype)
+    w_down = (torch.randn(width, n, generator=g) * ff ** -0.5).to(dtype)
+    ids = torch.stack([torch.randperm(E + ident, generator=g)[:top] for _ in range(T)]).to(torch.int32)
+    if ident:
+        ids[0, 0] = E + ident - 1                  # an identity expert in a fixed place too
+        ids[0, 1:] = torch.arange(top - 1)
+    w = torch.rand(T, top, generator=g) + 0.1
+    logits = torch.randn(T, E + ident + 1, generator=g)
+    sl = logits[:, E + ident] if shared else None
+    act_ref = torch.empty(T, top * ff + shared, dtype=dtype)
+    ref.moe_gate_up_chosen(x, w_gu, ids, w, act_ref, E, ff, shared, shared_logit=sl)
+    act = torch.full((T, top * ff + shared), float("nan"), dtype=dtype, device=DEV)
+    xd, idd, wd = x.to(DEV)[:, :], ids.to(DEV), w.to(DEV)
+    xd = torch.cat([torch.zeros(T, 8, dtype=dtype, device=DEV), xd], dim=1)[:, 8:]       # rows wider than the width
+    sld = logits.to(DEV)[:, E + ident] if shared else None
+    ops.moe_gate_up_chosen(xd, w_gu.to(DEV), idd, wd, act, E, ff, shared, shared_logit=sld)
+    close(act, act_ref, 2e-5 if dtype == torch.float32 else 1.5e-2, "act")
+    out_ref = torch.empty(T, width, dtype=dtype)
+    ref.moe_down_gated_chosen(act_ref, w_down, ids, w, x, out_ref, E, ff, shared)
+    out = torch.empty(T, width, dtype=dtype, device=DEV)
+    ops.moe_down_gated_chosen(act_ref.to(DEV), w_down.to(DEV), idd, wd, xd, out, E, ff, shared)
+    close(out, out_ref, 2e-5 if dtype == torch.float32 else 1.5e-2, "out")
+    # every expert through the products, the others' activations zero: the same sum
+    gu = torch.empty(T, 2 * n, dtype=dtype, device=DEV)
+    ops.linear(xd, w_gu.to(DEV), gu)
+    full = torch.empty(T, n, dtype=dtype, device=DEV)
+    ops.moe_silu_gate_scale(gu, full, idd, wd, E, ff, shared, shared_logit=sld)
+    dense = torch.empty(T, width, dtype=dtype, device=DEV)
+    ops.linear(full, w_down.to(DEV), dense)
+    ops.moe_identity_add(dense, xd, idd, wd, E)
+    close(out, dense.cpu(), 5e-5 if dtype == torch.float32 else 3e-2, "against every expert")
 
 
 @pytest.mark.parametrize("H,N,K", [(3, 24, 48), (8, 48, 96), (5, 8, 40), (2, 128, 576), (1, 7, 19)])
