@@ -287,12 +287,45 @@ __global__ void moe_identity_add_kernel(TA* __restrict__ y, int ldy, const TA* _
     y[t * ldy + e] = from_f32<TA>(to_f32(y[t * ldy + e]) + coef * to_f32(x[t * ldx + e]));
 }
 
+// the same, eight columns a thread through 16-byte accesses, a row split over blockIdx.y
+template <typename TA>
+__global__ void moe_identity_add_x8_kernel(TA* __restrict__ y, int ldy, const TA* __restrict__ x, int ldx,
+                                           const int* __restrict__ ids, const float* __restrict__ weights, int top,
+                                           int E, int width) {
+  const size_t t = blockIdx.x;
+  const int e = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
+  if (e >= width) return;
+  float coef = 0.f;
+  for (int j = 0; j < top; ++j)
+    if (ids[t * top + j] >= E) coef += weights[t * top + j];
+  if (coef == 0.f) return;
+  float a[8], b[8];
+  Vec8<TA>::load(y + t * ldy + e, a);
+  Vec8<TA>::load(x + t * ldx + e, b);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) a[i] += coef * b[i];
+  Vec8<TA>::store(y + t * ldy + e, a);
+}
+
 extern "C" int ra_moe_identity_add(void* y, int ldy, const void* x, int ldx, int act_dtype, const int* ids,
                                    const float* weights, int top, int experts, int n_tokens, int width,
                                    hipStream_t stream) {
   RA_CHECK(n_tokens > 0 && width > 0 && top > 0 && ldy >= width && ldx >= width,
            "moe_identity_add: %d tokens, width %d, %d choices", n_tokens, width, top);
   const int threads = width >= 1024 ? 256 : width >= 256 ? 128 : 64;
+  const int ab = act_dtype == RA_F32 ? 4 : 2;
+  if (width % 8 == 0 && ra_rows_16b(y, ldy, ab) && ra_rows_16b(x, ldx, ab) && (act_dtype == RA_F32 || act_dtype == RA_BF16)) {
+    const int vthreads = width >= 2048 ? 128 : 64;
+    const dim3 vgrid(n_tokens, (width / 8 + vthreads - 1) / vthreads);
+    if (act_dtype == RA_F32)
+      moe_identity_add_x8_kernel<float><<<vgrid, vthreads, 0, stream>>>((float*)y, ldy, (const float*)x, ldx, ids, weights,
+                                                                        top, experts, width);
+    else
+      moe_identity_add_x8_kernel<bf16_t><<<vgrid, vthreads, 0, stream>>>((bf16_t*)y, ldy, (const bf16_t*)x, ldx, ids,
+                                                                         weights, top, experts, width);
+    RA_LAUNCH_CHECK("moe_identity_add");
+    return 0;
+  }
   if (act_dtype == RA_F32)
     moe_identity_add_kernel<float><<<n_tokens, threads, 0, stream>>>((float*)y, ldy, (const float*)x, ldx, ids, weights,
                                                                      top, experts, width);
