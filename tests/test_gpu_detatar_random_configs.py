@@ -21,14 +21,23 @@ from reinfer_amd.weights.safetensors_io import write_safetensors
 pytestmark = pytest.mark.gpu
 
 
-def draw_config(rng: random.Random) -> dict:
-    groups = rng.choice([1, 1, 2, 3, 4])
-    width = groups * rng.choice([8, 12, 24, 40])
+def draw_config(rng: random.Random, wide: bool = False) -> dict:
+    """``wide``: sizes of a larger model's (heads of 96 and 128, latents of 256 and 512, dozens of experts)."""
+    groups = rng.choice([1, 1, 2, 3, 4] if not wide else [1, 2, 4, 8, 6])
+    width = groups * rng.choice([8, 12, 24, 40] if not wide else [32, 48, 64, 100])
 
     def wkv():
+        if wide:
+            return {"dim": rng.choice([48, 64, 96, 128]), "heads": rng.choice([2, 4, 6, 8])}
         return {"dim": rng.choice([4, 9, 16, 32, 40, 64, 72]), "heads": rng.choice([1, 2, 3, 5])}
 
     def latent():
+        if wide:
+            rot_dim = rng.choice([16, 32, 64, 128])
+            return {"dim": rng.choice([32, 48, 64, 96, 128]), "heads": rng.choice([2, 6, 8, 12, 16, 32]),
+                    "kv_rank": rng.choice([48, 96, 160, 256, 512]), "q_rank": rng.choice([24, 80, 200, 384]),
+                    "rot_dim": rot_dim, "scale": rng.choice([0.05, 0.1, 0.2]), "vdim": rng.choice([16, 40, 64, 96, 128]),
+                    "rot": {"base": rng.choice([100.0, 10000.0, 1e6]), "dims": rot_dim}}
         rot_dim = rng.choice([2, 4, 8, 16, 32, 64])
         m = {"dim": rng.choice([0, 8, 16, 24, 32, 64]), "heads": rng.choice([1, 2, 3, 4, 8, 16]),
              "kv_rank": rng.choice([8, 24, 32, 64, 128]), "q_rank": rng.choice([4, 12, 48]), "rot_dim": rot_dim,
@@ -42,8 +51,8 @@ def draw_config(rng: random.Random) -> dict:
             return None
         if kind == "dense":
             return {"ff": rng.choice([16, 40, 100]), "kind": "dense"}
-        count = rng.choice([1, 2, 3, 5])
-        per = rng.choice([1, 2, 4])
+        count = rng.choice([1, 2, 3, 5] if not wide else [2, 4, 8])
+        per = rng.choice([1, 2, 4] if not wide else [3, 4, 8])
         keep = rng.randint(1, count)
         routed = count * per
         identity = rng.choice([0, 0, 1, 2, 3])
@@ -81,10 +90,11 @@ def draw_config(rng: random.Random) -> dict:
     return raw
 
 
-@pytest.mark.parametrize("seed,dtype", [(s, "float32") for s in range(20)] + [(s, "bfloat16") for s in range(20, 30)])
+@pytest.mark.parametrize("seed,dtype", [(s, "float32") for s in range(20)] + [(s, "bfloat16") for s in range(20, 30)]
+                         + [(s, "float32") for s in range(100, 110)] + [(s, "bfloat16") for s in range(110, 114)])
 def test_random_configuration(tmp_path, seed, dtype):
     rng = random.Random(2000 + seed)
-    raw = draw_config(rng)
+    raw = draw_config(rng, wide=seed >= 100)
     if dtype == "bfloat16":
         for L in raw["layers"]:
             if L["mlp"] is not None and L["mlp"]["kind"] == "moe":
