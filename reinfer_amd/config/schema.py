@@ -93,6 +93,7 @@ class NormSpec:
     eps: float
     offset: float = 0.0  # the stored weight lies around zero: the factor is offset + w (1.0 for "one plus w")
     groups: int = 1      # the row is normed in this many equal consecutive parts, each over its own root mean square
+    scalar: bool = False # the stored weight is one number that multiplies every coordinate
 
 
 @dataclass(frozen=True)
@@ -125,6 +126,13 @@ class MixerSpec:
     # A mixer that is not attention-shaped brings a record of its own (any frozen dataclass) with the
     # sizes and constants it needs, typed as it likes; the fields above then stay at their defaults.
     params: Any = None
+    # further options of attention
+    qk_norm_whole: bool = False     # q and k are normed over their whole projection (all heads at once), weights of that size
+    softcap: float = 0.0            # score <- softcap * tanh(score / softcap) when > 0
+    distance_bias: bool = False     # score -= r1_h * ln(1 + r2_h * (i - j)), two numbers a query head
+    rotate_values: bool = False     # a value is turned by its own position over its whole size, a head's result back by the query's
+    out_gate: bool = False          # the concatenated heads times sigmoid(W_g h), element by element, before the output projection
+    kv_shared: bool = False         # the mixer has no key and value tensors: it reads another run entry's cache
 
     def option(self, name: str, default: Any = None) -> Any:
         return dict(self.extra).get(name, default)
@@ -170,7 +178,9 @@ class MoESpec:
     ``weights`` "softmax": scores are the softmax over all router outputs, the choice is by score plus a stored
     correction (``correction``) inside the best groups (``group_top`` 1: a group's score is its largest choice
     score), the weights the chosen scores over their sum + ``norm_eps``. ``identity`` > 0: that many further
-    router outputs behind the experts stand for experts without matrices whose output is their input."""
+    router outputs behind the experts stand for experts without matrices whose output is their input.
+    ``weights`` "table": no router; an integer table [vocabulary, top] gives each token id its experts, each
+    weighing 1 / top."""
     experts: int
     top: int
     activation: str = "relu2"
@@ -198,6 +208,19 @@ class MatrixMemorySpec:
     gate_cap: float
     norm_eps: float
     denom_eps: float = 1e-6
+
+
+@dataclass(frozen=True)
+class DecayMemorySpec:
+    """A matrix state a head that fades by a constant a head (``MixerSpec.params`` of the "decay_memory" mixer):
+    S <- decays[h] * S + k v^T, o = S^T q, with ``heads`` heads of ``key_dim`` x ``value_dim`` and silu on q, k and
+    v; the concatenated read-outs are RMS-normed together (``norm_eps``), times a plain weight and a sigmoid
+    gate."""
+    heads: int
+    key_dim: int
+    value_dim: int
+    decays: Tuple[float, ...]
+    norm_eps: float
 
 
 @dataclass(frozen=True)
@@ -248,6 +271,9 @@ class SideBySideSpec:
     members: Tuple[Tuple[str, Any], ...]
     norm_eps: float
     out_name: str = "out"
+    # "normed_mean" as above; "scaled_sum": y = sum_i scales[i] * mixer_i(h), no norms and no weights
+    combine: str = "normed_mean"
+    scales: Tuple[float, ...] = ()
 
 
 @dataclass(frozen=True)

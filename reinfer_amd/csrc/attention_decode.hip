@@ -66,7 +66,8 @@ __device__ __forceinline__ FdCut fd_cut(int p, int lo, int chunk_shift, int max_
 }
 
 // EXACT: the head size is DMAX itself, so every test against it is decided when the kernel is compiled
-template <int DMAX, bool EXACT, int FD_WAVES>
+// MOD: the scores are changed before the softmax (RaScoreMod: a tanh cap, a per-head distance term)
+template <int DMAX, bool EXACT, int FD_WAVES, bool MOD>
 __global__ void __launch_bounds__(FD_WAVES * RA_WAVE, (DMAX <= 128 && FD_WAVES == 4) ? 3 : 1)
 flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
                     const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
@@ -74,7 +75,7 @@ flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restri
                     const int* __restrict__ token_list, const int* __restrict__ seq_of_token,
                     const int* __restrict__ positions, int block_size, int Hkv, int G, int d_arg,
                     float scale_log2, int window, int chunk_shift, int max_chunks, int n_tokens,
-                    int t_base, float* __restrict__ part_o, float* __restrict__ part_ml) {
+                    int t_base, float* __restrict__ part_o, float* __restrict__ part_ml, float scale, RaScoreMod mod) {
   constexpr int FD_THREADS = FD_WAVES * RA_WAVE;
   const int d = EXACT ? DMAX : d_arg;
   constexpr int NDT = DMAX / 32;       // 32-wide d tiles of the score product
@@ -114,6 +115,10 @@ flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restri
 #pragma unroll
     for (int i = 0; i < NOT; ++i) acc[i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
+    // the distance term's two numbers of this lane's query head (column r)
+    const bool biased = MOD && mod.r1 != nullptr;
+    const float r1h = (biased && r < G) ? mod.r1[kvh * G + r] : 0.f;
+    const float r2h = (biased && r < G) ? mod.r2[kvh * G + r] : 0.f;
 
     const int k_begin = cut.base + ci * cut.chunk;
     const int k_end = min(k_begin + cut.chunk, p + 1);
@@ -178,7 +183,11 @@ flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restri
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int key = k0 + tt * 16 + 4 * g + i;
-          const float v = (key <= p && key >= lo) ? s[tt][i] * scale_log2 : -INFINITY;
+          float v = -INFINITY;
+          if (key <= p && key >= lo) {
+            if (MOD) v = ra_mod_score(s[tt][i] * scale, mod.softcap, biased, r1h, r2h, p - key) * 1.4426950408889634f;
+            else v = s[tt][i] * scale_log2;
+          }
           s[tt][i] = v;
           tmax = fmaxf(tmax, v);
         }
@@ -401,7 +410,10 @@ static size_t fd_lds_limit(void) {
 template <int DM, bool EX, int WV>
 static hipError_t fd_allow_lds(size_t lds) {
   if (lds <= 64 * 1024) return hipSuccess;
-  return hipFuncSetAttribute((const void*)flash_decode_kernel<DM, EX, WV>, hipFuncAttributeMaxDynamicSharedMemorySize,
+  hipError_t e = hipFuncSetAttribute((const void*)flash_decode_kernel<DM, EX, WV, false>,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return e;
+  return hipFuncSetAttribute((const void*)flash_decode_kernel<DM, EX, WV, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
                              (int)lds);
 }
 
@@ -418,8 +430,8 @@ static int fd_resident_workgroups(int variant, int waves, size_t lds) {
 #define RA_FD_OCC(DM)                                                                                                  \
   e = waves == 4 ? fd_allow_lds<DM, true, 4>(lds) : fd_allow_lds<DM, true, 12>(lds);                                   \
   if (e == hipSuccess)                                                                                                 \
-  e = waves == 4 ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, flash_decode_kernel<DM, true, 4>, 4 * RA_WAVE, lds) \
-                 : hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, flash_decode_kernel<DM, true, 12>, 12 * RA_WAVE, lds)
+  e = waves == 4 ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, flash_decode_kernel<DM, true, 4, false>, 4 * RA_WAVE, lds) \
+                 : hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, flash_decode_kernel<DM, true, 12, false>, 12 * RA_WAVE, lds)
   if (variant == 0) RA_FD_OCC(64);
   else if (variant == 1) RA_FD_OCC(128);
   else RA_FD_OCC(256);
@@ -458,6 +470,24 @@ extern "C" int ra_attention_decode(const void* q, int q_stride, void* out, int o
                                    const int* positions, int n_tokens, int block_size, int Hq, int Hkv,
                                    int d, float scale, int window, int chunk, int max_chunks, int waves,
                                    float* part_o, float* part_ml, hipStream_t stream) {
+  return ra_attention_decode_mod(q, q_stride, out, out_stride, kcache, vcache, block_tables, max_blocks, token_list,
+                                 seq_of_token, positions, n_tokens, block_size, Hq, Hkv, d, scale, window, chunk,
+                                 max_chunks, waves, part_o, part_ml, 0.f, nullptr, nullptr, stream);
+}
+
+// The same with the scores changed before the softmax: softcap > 0 caps them by a tanh, r1 / r2 (one float a query
+// head each; both or neither) take r1 ln(1 + r2 (position - key)) off.
+extern "C" int ra_attention_decode_mod(const void* q, int q_stride, void* out, int out_stride,
+                                       const void* kcache, const void* vcache, const int* block_tables,
+                                       int max_blocks, const int* token_list, const int* seq_of_token,
+                                       const int* positions, int n_tokens, int block_size, int Hq, int Hkv,
+                                       int d, float scale, int window, int chunk, int max_chunks, int waves,
+                                       float* part_o, float* part_ml, float softcap, const float* r1,
+                                       const float* r2, hipStream_t stream) {
+  RA_CHECK((r1 == nullptr) == (r2 == nullptr) && softcap >= 0.f,
+           "attention_decode: the distance term takes both per-head vectors, the cap is not negative");
+  const RaScoreMod mod = {softcap, r1, r2};
+  const bool changed = softcap > 0.f || r1 != nullptr;
   RA_CHECK(n_tokens > 0, "attention_decode: no tokens");
   RA_CHECK(ra_attention_decode_supports(Hq, Hkv, d, block_size),
            "attention_decode: unsupported sizes (%d query heads, %d KV heads, head size %d, block %d)", Hq,
@@ -483,14 +513,16 @@ extern "C" int ra_attention_decode(const void* q, int q_stride, void* out, int o
   const long items_max = (long)n_tokens * Hkv * max_chunks;
   RA_CHECK(items_max < (1L << 30), "attention_decode: %ld work items in one launch", items_max);
   const int grid = (int)(items_max < slots ? items_max : slots);
+#define RA_FD_ARGS                                                                                    \
+  (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache, (const bf16_t*)vcache, \
+      block_tables, max_blocks, token_list, seq_of_token, positions, block_size, Hkv, G, d, scale_log2, \
+      window, chunk_shift, max_chunks, n_tokens, 0, part_o, part_ml, scale, mod
 #define RA_FD_GO(DM, EX, WV)                                                                          \
   do {                                                                                                \
     if (fd_allow_lds<DM, EX, WV>(lds) != hipSuccess)                                                  \
       return ra_fail("attention_decode: the device does not give a workgroup %zu bytes of LDS", lds); \
-    flash_decode_kernel<DM, EX, WV><<<grid, WV * RA_WAVE, lds, stream>>>(                             \
-        (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,                  \
-        (const bf16_t*)vcache, block_tables, max_blocks, token_list, seq_of_token, positions, block_size, \
-        Hkv, G, d, scale_log2, window, chunk_shift, max_chunks, n_tokens, 0, part_o, part_ml);        \
+    if (changed) flash_decode_kernel<DM, EX, WV, true><<<grid, WV * RA_WAVE, lds, stream>>>(RA_FD_ARGS); \
+    else flash_decode_kernel<DM, EX, WV, false><<<grid, WV * RA_WAVE, lds, stream>>>(RA_FD_ARGS);     \
   } while (0)
 #define RA_FD(DM)                                                                                     \
   do {                                                                                                \
@@ -507,6 +539,7 @@ extern "C" int ra_attention_decode(const void* q, int q_stride, void* out, int o
   else RA_FD(256);
 #undef RA_FD_GO
 #undef RA_FD
+#undef RA_FD_ARGS
   RA_LAUNCH_CHECK("attention_decode");
   if (max_chunks > 1) {
     RA_CHECK(n_tokens <= 65535, "attention_decode: %d tokens in one launch of the merge (max 65535)", n_tokens);

@@ -7,6 +7,8 @@
 //   lo = max(0, p - window + 1) if window > 0 else 0; softmax with the running
 //   maximum subtracted; o = sum_t P_t V_t.
 //   Query head a reads KV head a / (Hq / Hkv).
+//   With a score change (RaScoreMod): s <- cap tanh(s / cap) where cap > 0, then
+//   s <- s - r1[a] ln(1 + r2[a] (p - t)) where the two per-head vectors are given.
 // (crates/cuda/kernels/decode_gqa_kernels.cu:69-136; plain form
 //  crates/cuda/tests/engine_vs_cpu.rs:205-241)
 #include "common.h"
@@ -20,7 +22,7 @@ __global__ void attention_plain_kernel(const TA* __restrict__ q, int q_stride, T
                                        const int* __restrict__ token_list,
                                        const int* __restrict__ seq_of_token,
                                        const int* __restrict__ positions, int block_size, int Hq,
-                                       int Hkv, int d, float scale, int window) {
+                                       int Hkv, int d, float scale, int window, RaScoreMod mod) {
   extern __shared__ float lds[];          // q vector [d], then probabilities [64]
   float* qs = lds;
   float* ps = lds + d;
@@ -51,7 +53,8 @@ __global__ void attention_plain_kernel(const TA* __restrict__ q, int q_stride, T
       const int off = key % block_size;
       float dot = 0.f;
       for (int i = 0; i < d; ++i) dot += qs[i] * to_f32(kr[cache_k_index(off, i, d)]);
-      s = dot * scale;
+      s = ra_mod_score(dot * scale, mod.softcap, mod.r1 != nullptr, mod.r1 ? mod.r1[a] : 0.f, mod.r1 ? mod.r2[a] : 0.f,
+                       p - key);
     }
     const float cmax = wave_max(s);
     const float m_new = fmaxf(m, cmax);
@@ -96,6 +99,20 @@ extern "C" int ra_attention_plain(const void* q, int q_stride, void* out, int ou
                                   const int* block_tables, int max_blocks, const int* token_list,
                                   const int* seq_of_token, const int* positions, int n_tokens, int block_size, int Hq, int Hkv,
                                   int d, float scale, int window, hipStream_t stream) {
+  return ra_attention_plain_mod(q, q_stride, out, out_stride, kcache, vcache, act_dtype, block_tables, max_blocks,
+                                token_list, seq_of_token, positions, n_tokens, block_size, Hq, Hkv, d, scale, window,
+                                0.f, nullptr, nullptr, stream);
+}
+
+extern "C" int ra_attention_plain_mod(const void* q, int q_stride, void* out, int out_stride,
+                                      const void* kcache, const void* vcache, int act_dtype,
+                                      const int* block_tables, int max_blocks, const int* token_list,
+                                      const int* seq_of_token, const int* positions, int n_tokens, int block_size,
+                                      int Hq, int Hkv, int d, float scale, int window, float softcap,
+                                      const float* r1, const float* r2, hipStream_t stream) {
+  RA_CHECK((r1 == nullptr) == (r2 == nullptr) && softcap >= 0.f,
+           "attention_plain: the distance term takes both per-head vectors, the cap is not negative");
+  const RaScoreMod mod = {softcap, r1, r2};
   RA_CHECK(n_tokens > 0, "attention_plain: no tokens");
   RA_CHECK(Hq > 0 && Hkv > 0 && Hq % Hkv == 0, "attention_plain: %d query heads do not divide into %d groups", Hq, Hkv);
   RA_CHECK(d > 0 && d <= 1024, "attention_plain: head size %d outside 1..1024", d);
@@ -109,12 +126,12 @@ extern "C" int ra_attention_plain(const void* q, int q_stride, void* out, int ou
   if (act_dtype == RA_F32)
     attention_plain_kernel<float><<<grid, RA_WAVE, lds, stream>>>(
         (const float*)q, q_stride, (float*)out, out_stride, (const float*)kcache, (const float*)vcache,
-        block_tables, max_blocks, token_list, seq_of_token, positions, block_size, Hq, Hkv, d, scale, window);
+        block_tables, max_blocks, token_list, seq_of_token, positions, block_size, Hq, Hkv, d, scale, window, mod);
   else if (act_dtype == RA_BF16)
     attention_plain_kernel<bf16_t><<<grid, RA_WAVE, lds, stream>>>(
         (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,
         (const bf16_t*)vcache, block_tables, max_blocks, token_list, seq_of_token, positions, block_size,
-        Hq, Hkv, d, scale, window);
+        Hq, Hkv, d, scale, window, mod);
   else
     return ra_fail("attention_plain: unknown dtype tag %d", act_dtype);
   RA_LAUNCH_CHECK("attention_plain");

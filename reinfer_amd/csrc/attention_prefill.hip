@@ -68,14 +68,16 @@ struct FpSplit {
 };
 
 // EXACT: the head size is DMAX itself, so every test against it is decided when the kernel is compiled
-template <int DMAX, int NC, bool EXACT>
+// MOD: the scores are changed before the softmax (RaScoreMod: a tanh cap, a per-head distance term); the scaled
+// and changed score then replaces the product in the registers, and scale_log2 is log2(e) alone
+template <int DMAX, int NC, bool EXACT, bool MOD>
 __global__ void __launch_bounds__(FP_THREADS)
 flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
                      const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
                      const int* __restrict__ block_tables, int max_blocks,
                      const int* __restrict__ tile_info,      // per tile: seq, first token row, n queries, first position
                      int block_size, int Hq, int Hkv, int d_arg, int HG, float scale_log2, int window,
-                     FpSplit sp) {
+                     FpSplit sp, float mod_scale, RaScoreMod mod) {
   const int d = EXACT ? DMAX : d_arg;
   constexpr int NDT = DMAX / 32;       // 32-wide d tiles of the score product
   constexpr int NOT = DMAX / 16;       // 16-row d tiles of the output
@@ -114,12 +116,16 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
   int qi[NC];
   bool q_live[NC];
   bf16x8_t qreg[NC][NDT];
+  const bool biased = MOD && mod.r1 != nullptr;
+  float r1h[NC], r2h[NC];               // the distance term's two numbers of each column tile's head
 #pragma unroll
   for (int j = 0; j < NC; ++j) {
     const int c = wave * NC + j;
     qi[j] = (c / HG) * 16 + r;
     q_live[j] = qi[j] < nq && ((col_mask >> j) & 1);
     const int head = kvh * G + hgrp * HG + c % HG;
+    r1h[j] = biased ? mod.r1[head] : 0.f;
+    r2h[j] = biased ? mod.r2[head] : 0.f;
     const bf16_t* qp = q + (size_t)(row0 + (q_live[j] ? qi[j] : 0)) * q_stride + (size_t)head * d;
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) {
@@ -291,6 +297,20 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
       if (NC == 1 || col_mask == (1 << NC) - 1) scores(I0{}, IN{});
       else if (col_mask == 1) scores(I0{}, I1{});
       else scores(I1{}, IN{});
+      if constexpr (MOD) {
+        // a key past the query (masked below) counts as distance 0: its changed score is never used
+#pragma unroll
+        for (int j = 0; j < NC; ++j) {
+          const int q_pos = pos0 + qi[j];
+#pragma unroll
+          for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int key = kh + ks * 16 + 4 * g + i;
+              s[ks][j][i] = ra_mod_score(s[ks][j][i] * mod_scale, mod.softcap, biased, r1h[j], r2h[j], max(q_pos - key, 0));
+            }
+        }
+      }
       // keys strictly inside every query's view need no mask
       const bool inner = kh + 31 <= w_first_pos && w_qend <= nq &&
                          (window <= 0 || kh >= w_last_pos - window + 1);
@@ -559,7 +579,10 @@ static int fp_launch(const void* q, int q_stride, void* out, int out_stride,
                      const void* kcache, const void* vcache, const int* block_tables,
                      int max_blocks, const int* tile_info, int n_tiles, int block_size,
                      int Hq, int Hkv, int d, float scale, int window, const FpSplit& sp, const int* merge_info,
-                     int n_merge, hipStream_t stream) {
+                     int n_merge, const RaScoreMod& mod, hipStream_t stream) {
+  RA_CHECK((mod.r1 == nullptr) == (mod.r2 == nullptr) && mod.softcap >= 0.f,
+           "attention_prefill: the distance term takes both per-head vectors, the cap is not negative");
+  const bool changed = mod.softcap > 0.f || mod.r1 != nullptr;
   RA_CHECK(n_tiles > 0, "attention_prefill: no query tiles");
   RA_CHECK(ra_attention_prefill_supports(Hq, Hkv, d, block_size),
            "attention_prefill: unsupported sizes (%d query heads, %d KV heads, head size %d, block %d)", Hq,
@@ -574,12 +597,15 @@ static int fp_launch(const void* q, int q_stride, void* out, int out_stride,
   RA_CHECK(gy <= 65535, "attention_prefill: too many heads for one launch");
   RA_CHECK((long)n_tiles * gy <= 0x7fffffffL, "attention_prefill: too many workgroups");
   dim3 grid(n_tiles * gy);
-  const float scale_log2 = scale * 1.4426950408889634f;
+  const float scale_log2 = (changed ? 1.f : scale) * 1.4426950408889634f;
+#define RA_FP_ARGS                                                                                    \
+  (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache, (const bf16_t*)vcache, \
+      block_tables, max_blocks, tile_info, block_size, Hq, Hkv, d, sh.hg, scale_log2, window, sp, scale, mod
 #define RA_FP_GO(DM, NCC, EX)                                                                         \
-  flash_prefill_kernel<DM, NCC, EX><<<grid, FP_THREADS, 0, stream>>>(                                 \
-      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,                    \
-      (const bf16_t*)vcache, block_tables, max_blocks, tile_info, block_size, Hq, Hkv, d, sh.hg,      \
-      scale_log2, window, sp)
+  do {                                                                                                \
+    if (changed) flash_prefill_kernel<DM, NCC, EX, true><<<grid, FP_THREADS, 0, stream>>>(RA_FP_ARGS); \
+    else flash_prefill_kernel<DM, NCC, EX, false><<<grid, FP_THREADS, 0, stream>>>(RA_FP_ARGS);       \
+  } while (0)
 #define RA_FP(DM, NCC)                                                                                \
   do {                                                                                                \
     if (d == DM && DM <= 128) RA_FP_GO(DM, NCC, true); /* at 256 the exact form spills registers */   \
@@ -590,6 +616,7 @@ static int fp_launch(const void* q, int q_stride, void* out, int out_stride,
   else RA_FP(256, 1);
 #undef RA_FP_GO
 #undef RA_FP
+#undef RA_FP_ARGS
   RA_LAUNCH_CHECK("attention_prefill");
   if (n_merge > 0) {
     const int n_cols = FP_WAVES * sh.nc * 16;
@@ -610,9 +637,21 @@ extern "C" int ra_attention_prefill(const void* q, int q_stride, void* out, int 
                                     const void* kcache, const void* vcache, const int* block_tables,
                                     int max_blocks, const int* tile_info, int n_tiles, int block_size,
                                     int Hq, int Hkv, int d, float scale, int window, hipStream_t stream) {
+  return ra_attention_prefill_mod(q, q_stride, out, out_stride, kcache, vcache, block_tables, max_blocks, tile_info,
+                                  n_tiles, block_size, Hq, Hkv, d, scale, window, 0.f, nullptr, nullptr, stream);
+}
+
+// The same with the scores changed before the softmax: softcap > 0 caps them by a tanh, r1 / r2 (one float a query
+// head each; both or neither) take r1 ln(1 + r2 (position - key)) off.
+extern "C" int ra_attention_prefill_mod(const void* q, int q_stride, void* out, int out_stride,
+                                        const void* kcache, const void* vcache, const int* block_tables,
+                                        int max_blocks, const int* tile_info, int n_tiles, int block_size,
+                                        int Hq, int Hkv, int d, float scale, int window, float softcap,
+                                        const float* r1, const float* r2, hipStream_t stream) {
   const FpSplit none = {};
+  const RaScoreMod mod = {softcap, r1, r2};
   return fp_launch(q, q_stride, out, out_stride, kcache, vcache, block_tables, max_blocks, tile_info, n_tiles,
-                   block_size, Hq, Hkv, d, scale, window, none, nullptr, 0, stream);
+                   block_size, Hq, Hkv, d, scale, window, none, nullptr, 0, mod, stream);
 }
 
 // The same with query tiles cut by keys: `ranges` holds three ints a listed tile (first key and one past the
@@ -625,6 +664,18 @@ extern "C" int ra_attention_prefill_split(const void* q, int q_stride, void* out
                                           const int* merge_info, int n_merge, float* part_o, float* part_ml,
                                           int block_size, int Hq, int Hkv, int d, float scale, int window,
                                           hipStream_t stream) {
+  return ra_attention_prefill_split_mod(q, q_stride, out, out_stride, kcache, vcache, block_tables, max_blocks,
+                                        tile_info, n_tiles, ranges, merge_info, n_merge, part_o, part_ml, block_size,
+                                        Hq, Hkv, d, scale, window, 0.f, nullptr, nullptr, stream);
+}
+
+extern "C" int ra_attention_prefill_split_mod(const void* q, int q_stride, void* out, int out_stride,
+                                              const void* kcache, const void* vcache, const int* block_tables,
+                                              int max_blocks, const int* tile_info, int n_tiles, const int* ranges,
+                                              const int* merge_info, int n_merge, float* part_o, float* part_ml,
+                                              int block_size, int Hq, int Hkv, int d, float scale, int window,
+                                              float softcap, const float* r1, const float* r2, hipStream_t stream) {
+  const RaScoreMod mod = {softcap, r1, r2};
   RA_CHECK(ranges && merge_info && n_merge > 0 && part_o && part_ml,
            "attention_prefill_split: ranges, the list of cut tiles and the buffers for their parts are needed");
   RA_CHECK(((uintptr_t)part_o % 16) == 0, "attention_prefill_split: the parts' buffer must be 16-byte aligned");
@@ -633,5 +684,5 @@ extern "C" int ra_attention_prefill_split(const void* q, int q_stride, void* out
   sp.part_o = part_o;
   sp.part_ml = part_ml;
   return fp_launch(q, q_stride, out, out_stride, kcache, vcache, block_tables, max_blocks, tile_info, n_tiles,
-                   block_size, Hq, Hkv, d, scale, window, sp, merge_info, n_merge, stream);
+                   block_size, Hq, Hkv, d, scale, window, sp, merge_info, n_merge, mod, stream);
 }

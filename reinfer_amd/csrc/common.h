@@ -85,6 +85,20 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
   return t;
 }
 
+// ---- what attention does to a score between the scaled product and the softmax -------------------------------
+// softcap > 0: s <- softcap * tanh(s / softcap); r1, r2 (float, one entry a query head; both or neither):
+// s <- s - r1[h] * ln(1 + r2[h] * (query position - key position)). The cap comes first.
+struct RaScoreMod {
+  float softcap;
+  const float* r1;
+  const float* r2;
+};
+__device__ __forceinline__ float ra_mod_score(float s, float softcap, bool biased, float r1, float r2, int dist) {
+  if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+  if (biased) s -= r1 * logf(1.f + r2 * (float)dist);
+  return s;
+}
+
 // ---- cache layout -----------------------------------------------------------
 // A block of the cache holds block_size (a multiple of 16) slots of one KV head
 // as block_size/16 tiles of 16 slots x d elements, 16*d elements each, laid out

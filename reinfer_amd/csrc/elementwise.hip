@@ -902,15 +902,23 @@ extern "C" int ra_qk_norm_rope_cache_sums(const float* parts, int n_ranges, cons
 // group == 0 gate is columns [0, I) and up [I, 2I); with group > 0 the two are
 // interleaved in runs of `group` columns, as the gated product kernel wants them.
 // ---------------------------------------------------------------------------
-// act 0: silu; act 1: the tanh form of gelu, 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
-__device__ __forceinline__ float gate_act(float g, int act) {
+// act 0: silu; act 1: the tanh form of gelu, 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)));
+// act 2: both inputs bounded by `lim` (the gate from above, the other from both sides), then
+// g sigmoid(1.702 g) (u + 1)
+__device__ __forceinline__ float gated_value(float g, float u, int act, float lim) {
   // 0.5 (1 + tanh y) = 1 / (1 + exp(-2 y))
-  if (act == 1) return g / (1.f + expf(-1.5957691216057308f * (g + 0.044715f * g * g * g)));
-  return g / (1.f + expf(-g));
+  if (act == 1) return g / (1.f + expf(-1.5957691216057308f * (g + 0.044715f * g * g * g))) * u;
+  if (act == 2) {
+    g = fminf(g, lim);
+    u = fminf(fmaxf(u, -lim), lim);
+    return g / (1.f + expf(-1.702f * g)) * (u + 1.f);
+  }
+  return g / (1.f + expf(-g)) * u;
 }
 
 template <typename TA>
-__global__ void silu_mul_kernel(const TA* __restrict__ gu, TA* __restrict__ out, int I, int group, size_t total, int act) {
+__global__ void silu_mul_kernel(const TA* __restrict__ gu, TA* __restrict__ out, int I, int group, size_t total, int act,
+                                float lim) {
   size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   for (; idx < total; idx += stride) {
@@ -920,13 +928,14 @@ __global__ void silu_mul_kernel(const TA* __restrict__ gu, TA* __restrict__ out,
     const size_t ui = group > 0 ? gi + group : (size_t)I + i;
     const float g = to_f32(gu[t * 2 * I + gi]);
     const float u = to_f32(gu[t * 2 * I + ui]);
-    out[idx] = from_f32<TA>(gate_act(g, act) * u);
+    out[idx] = from_f32<TA>(gated_value(g, u, act, lim));
   }
 }
 
 // eight outputs a thread, 16-byte loads and stores; I a multiple of 8, group 0 or a multiple of 8
 template <typename TA>
-__global__ void silu_mul_vec_kernel(const TA* __restrict__ gu, TA* __restrict__ out, int I, int group, size_t total8, int act) {
+__global__ void silu_mul_vec_kernel(const TA* __restrict__ gu, TA* __restrict__ out, int I, int group, size_t total8, int act,
+                                    float lim) {
   size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   const int I8 = I / 8;
@@ -940,8 +949,8 @@ __global__ void silu_mul_vec_kernel(const TA* __restrict__ gu, TA* __restrict__ 
     f32x4_raw u0 = Vec4<TA>::load(row + ui), u1 = Vec4<TA>::load(row + ui + 4);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      g0[e] = gate_act(g0[e], act) * u0[e];
-      g1[e] = gate_act(g1[e], act) * u1[e];
+      g0[e] = gated_value(g0[e], u0[e], act, lim);
+      g1[e] = gated_value(g1[e], u1[e], act, lim);
     }
     Vec4<TA>::store(out + idx * 8, g0);
     Vec4<TA>::store(out + idx * 8 + 4, g1);
@@ -955,8 +964,15 @@ extern "C" int ra_silu_mul(const void* gate_up, void* out, int act_dtype, int n_
 
 extern "C" int ra_act_mul(const void* gate_up, void* out, int act_dtype, int n_tokens, int intermediate,
                           int group, int act, hipStream_t stream) {
+  return ra_act_mul_bounded(gate_up, out, act_dtype, n_tokens, intermediate, group, act, 0.f, stream);
+}
+
+// `lim`: the bound of activation 2 (unused by the others)
+extern "C" int ra_act_mul_bounded(const void* gate_up, void* out, int act_dtype, int n_tokens, int intermediate,
+                                  int group, int act, float lim, hipStream_t stream) {
   RA_CHECK(n_tokens > 0 && intermediate > 0, "silu_mul: empty input");
-  RA_CHECK(act == 0 || act == 1, "act_mul: unknown activation %d", act);
+  RA_CHECK(act >= 0 && act <= 2, "act_mul: unknown activation %d", act);
+  RA_CHECK(act != 2 || lim > 0.f, "act_mul: the bounded activation needs a positive bound");
   RA_CHECK(group >= 0 && (group == 0 || intermediate % group == 0),
            "silu_mul: width %d is not a whole number of runs of %d", intermediate, group);
   const size_t total = (size_t)n_tokens * intermediate;
@@ -966,18 +982,18 @@ extern "C" int ra_act_mul(const void* gate_up, void* out, int act_dtype, int n_t
     size_t vb = (total8 + 255) / 256;
     if (vb > 65535 * 4) vb = 65535 * 4;
     if (act_dtype == RA_F32)
-      silu_mul_vec_kernel<float><<<(unsigned)vb, 256, 0, stream>>>((const float*)gate_up, (float*)out, intermediate, group, total8, act);
+      silu_mul_vec_kernel<float><<<(unsigned)vb, 256, 0, stream>>>((const float*)gate_up, (float*)out, intermediate, group, total8, act, lim);
     else
-      silu_mul_vec_kernel<bf16_t><<<(unsigned)vb, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, intermediate, group, total8, act);
+      silu_mul_vec_kernel<bf16_t><<<(unsigned)vb, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, intermediate, group, total8, act, lim);
     RA_LAUNCH_CHECK("silu_mul");
     return 0;
   }
   size_t blocks = (total + 255) / 256;
   if (blocks > 65535 * 4) blocks = 65535 * 4;
   if (act_dtype == RA_F32)
-    silu_mul_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>((const float*)gate_up, (float*)out, intermediate, group, total, act);
+    silu_mul_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>((const float*)gate_up, (float*)out, intermediate, group, total, act, lim);
   else if (act_dtype == RA_BF16)
-    silu_mul_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, intermediate, group, total, act);
+    silu_mul_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, intermediate, group, total, act, lim);
   else
     return ra_fail("silu_mul: unknown dtype tag %d", act_dtype);
   RA_LAUNCH_CHECK("silu_mul");

@@ -816,3 +816,25 @@ extern "C" int ra_moe_down_gated_chosen(const void* act, const void* w_down, con
   RA_LAUNCH_CHECK("moe_down_gated_chosen");
   return 0;
 }
+
+// ---------------------------------------------------------------------------
+// No router: an integer table [vocabulary, top] gives each token id its experts; each weighs 1 / top.
+// ---------------------------------------------------------------------------
+__global__ void moe_table_route_kernel(const int* __restrict__ token_ids, const int* __restrict__ table, int top,
+                                       int* __restrict__ ids, float* __restrict__ weights, long total) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const long t = i / top;
+  const int j = (int)(i - t * top);
+  ids[i] = table[(size_t)token_ids[t] * top + j];
+  weights[i] = 1.f / (float)top;
+}
+
+extern "C" int ra_moe_table_route(const int* token_ids, const int* table, int top, int* ids, float* weights,
+                                  int n_tokens, hipStream_t stream) {
+  RA_CHECK(n_tokens > 0 && top > 0, "moe_table_route: %d tokens, %d choices", n_tokens, top);
+  const long total = (long)n_tokens * top;
+  moe_table_route_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(token_ids, table, top, ids, weights, total);
+  RA_LAUNCH_CHECK("moe_table_route");
+  return 0;
+}

@@ -20,7 +20,7 @@ struct ScanGeom {
 };
 
 // kind 0: matrix memory (S, the normaliser n once a wave, the running maximum m); kind 1: delta rule (S);
-// kind 2: wkv (S)
+// kind 2: wkv (S); kind 3: a memory that fades by a constant a head (S)
 bool scan_geom(int kind, int dk, int dv, ScanGeom* g) {
   if (dk <= 0 || dv <= 0 || dk > 512) return false;
   // at most 8 elements a lane: the per-token chain of multiply-adds stays short, and a head has enough waves to
@@ -70,13 +70,15 @@ __device__ __forceinline__ float logsigmoid_f(float x) { return -softplus_f(-x);
 //   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
 // computed from the state before the decay: a = S^T k, b = S^T q, kq = k . q in one butterfly, then
 // u = beta (v - g a), o = g b + u kq, S <- g S + k u.
+// A memory that fades by a constant (DECAY): no gates; q, k and v pass silu as they are staged (float);
+//   S <- head_decay[h] S + k v^T;  o = S^T q   (the read-out sees the token's own write)
 // ---------------------------------------------------------------------------
 #define SCAN_KQ_REGS 8         // k (and q) values a thread fetches for a chunk
 #define SCAN_V_REGS 2
 #define SCAN_CHUNK_MAX 16
 #define SCAN_LDS_FLOATS 6144   // of one of the two buffers
 
-enum { SCAN_DELTA = 0, SCAN_MEMORY = 1, SCAN_WKV = 2 };
+enum { SCAN_DELTA = 0, SCAN_MEMORY = 1, SCAN_WKV = 2, SCAN_DECAY = 3 };
 
 struct ScanArgs {
   const void* q; const void* k; const void* v;     // column 0 of each in row 0; rows ld elements apart
@@ -90,14 +92,15 @@ struct ScanArgs {
   float* out;
   // wkv: the decays' pre-activations, float [T, H dk] with rows ldw apart, their bias w0 [H dk] and the bonus u [H dk]
   const float* w; int ldw; const float* w0; const float* u;
+  const float* head_decay;                           // the fading memory: one factor a head
 };
 
 template <typename TA, int R, int NPL, int MODE>
 __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
-  constexpr bool MEMORY = MODE == SCAN_MEMORY, WKV = MODE == SCAN_WKV;
+  constexpr bool MEMORY = MODE == SCAN_MEMORY, WKV = MODE == SCAN_WKV, DECAY = MODE == SCAN_DECAY;
   constexpr int CPW = RA_WAVE / R;
   constexpr int PITCH = NPL + 4;                     // floats of a lane's run of k (or q) in LDS, padded
-  constexpr int NG = MEMORY ? 3 : WKV ? 0 : 2;       // gate values a token
+  constexpr int NG = MEMORY ? 3 : (WKV || DECAY) ? 0 : 2;       // gate values a token
   constexpr int NGD = NG ? NG : 1;
   constexpr int NV = WKV ? 3 : 2;                    // vectors over the key size a token: k, q and, for wkv, the decay
   extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -166,6 +169,10 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
       if (kq_t[j] < n && kq_e[j]) {
         fk[j] = to_f32(kg[row0 + kq_g[j]]);
         fq[j] = to_f32(qg[row0 + kq_g[j]]) * p.q_scale;
+        if (DECAY) {
+          fk[j] = fk[j] / (1.f + expf(-fk[j]));
+          fq[j] = fq[j] / (1.f + expf(-fq[j]));
+        }
       }
       if (WKV) {                                     // the decay exp(-exp(z + w0)), float from its pre-activation on
         fw[j] = 0.f;
@@ -174,7 +181,10 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
       }
     }
 #pragma unroll
-    for (int j = 0; j < SCAN_V_REGS; ++j) fv[j] = v_t[j] < n ? to_f32(vg[row0 + v_g[j]]) : 0.f;
+    for (int j = 0; j < SCAN_V_REGS; ++j) {
+      fv[j] = v_t[j] < n ? to_f32(vg[row0 + v_g[j]]) : 0.f;
+      if (DECAY) fv[j] = fv[j] / (1.f + expf(-fv[j]));
+    }
     fg = (NG && g_t < n) ? p.gates[(size_t)t0 * NG * H + g_g] : 0.f;
   };
   auto stage = [&](float* buf) {                     // registers -> LDS
@@ -195,6 +205,7 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
   };
   float* st = p.state + (size_t)slot * p.slot_stride + (size_t)(head * p.waves_per_head + (active ? w : 0)) * p.wave_floats;
   const bool zero = p.fresh[seq] != 0;
+  const float fade = DECAY ? p.head_decay[head] : 1.f;
   float S[NPL], nrm[NPL], bonus[NPL];
 #pragma unroll
   for (int i = 0; i < NPL; ++i) {
@@ -253,6 +264,14 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
             const float kv = x.k[i] * x.v;
             po[i & 1] += x.q[i] * (S[i] + bonus[i] * kv);
             S[i] = x.w[i] * S[i] + kv;
+          }
+          o = group_sum<R>(po[0] + po[1]);
+        } else if (DECAY) {
+          float po[2] = {0.f, 0.f};
+#pragma unroll
+          for (int i = 0; i < NPL; ++i) {
+            S[i] = fade * S[i] + x.k[i] * x.v;
+            po[i & 1] += S[i] * x.q[i];
           }
           o = group_sum<R>(po[0] + po[1]);
         } else {
@@ -715,6 +734,36 @@ extern "C" int ra_wkv_scan(const void* proj, int act_dtype, int ld, int r_off, i
   if (act_dtype == RA_F32) scan_dispatch<float, SCAN_WKV>(g, L, a, stream);
   else scan_dispatch<bf16_t, SCAN_WKV>(g, L, a, stream);
   RA_LAUNCH_CHECK("wkv_scan");
+  return 0;
+}
+
+// kind 3 of ra_scan_state_floats: S <- decays[h] S + k v^T, o = S^T q, with silu on q, k and v as they are read.
+extern "C" int ra_decay_scan(const void* proj, int act_dtype, int ld, int q_off, int k_off, int v_off,
+                             const float* decays, float* state, long slot_stride, const int* cu_tokens,
+                             const int* state_slots, const int* fresh, int n_seqs, int n_tokens, int max_q_len,
+                             int heads, int key_dim, int value_dim, float* out, hipStream_t stream) {
+  RA_CHECK(n_seqs > 0 && n_tokens > 0 && heads > 0, "decay_scan: %d requests, %d tokens, %d heads", n_seqs, n_tokens, heads);
+  RA_CHECK(decays != nullptr, "decay_scan: one factor a head is needed");
+  ScanGeom g;
+  RA_CHECK(scan_geom(3, key_dim, value_dim, &g), "decay_scan: heads of %d x %d (keys up to 512)", key_dim, value_dim);
+  RA_CHECK(slot_stride >= (long)heads * g.waves * g.wave_floats, "decay_scan: a state slot of %ld floats, need %ld",
+           slot_stride, (long)heads * g.waves * g.wave_floats);
+  RA_CHECK(heads <= 65535, "decay_scan: %d heads in one launch", heads);
+  RA_CHECK(act_dtype == RA_F32 || act_dtype == RA_BF16, "decay_scan: unknown dtype tag %d", act_dtype);
+  const ScanLaunch L = scan_launch(g, n_seqs, heads, max_q_len);
+  const size_t es = act_dtype == RA_F32 ? 4 : 2;
+  ScanArgs a = {};
+  a.q = (const char*)proj + (size_t)q_off * es;
+  a.k = (const char*)proj + (size_t)k_off * es;
+  a.v = (const char*)proj + (size_t)v_off * es;
+  a.ld = ld; a.q_heads = heads; a.gates = nullptr; a.state = state; a.slot_stride = slot_stride;
+  a.cu_tokens = cu_tokens; a.state_slots = state_slots; a.fresh = fresh;
+  a.H = heads; a.dk = key_dim; a.dv = value_dim; a.waves_per_head = g.waves; a.wave_floats = g.wave_floats;
+  a.chunk = L.chunk; a.q_scale = 1.f; a.denom_eps = 0.f; a.out = out;
+  a.head_decay = decays;
+  if (act_dtype == RA_F32) scan_dispatch<float, SCAN_DECAY>(g, L, a, stream);
+  else scan_dispatch<bf16_t, SCAN_DECAY>(g, L, a, stream);
+  RA_LAUNCH_CHECK("decay_scan");
   return 0;
 }
 

@@ -5,7 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define RA_ABI_VERSION 22
+#define RA_ABI_VERSION 23
 
 #ifdef __cplusplus
 extern "C" {
@@ -52,6 +52,17 @@ int ra_attention_plain(const void* q, int q_stride, void* out, int out_stride, c
                        const int* token_list, const int* seq_of_token, const int* positions, int n_tokens,
                        int block_size,
                        int Hq, int Hkv, int d, float scale, int window, hipStream_t stream);
+// The `_mod` forms of the three attention kernels change a score between the scaled product and the softmax:
+// softcap > 0: s <- softcap tanh(s / softcap); r1, r2 (float, one entry a query head, both or neither):
+// s <- s - r1[h] ln(1 + r2[h] (query position - key position)); the cap first.
+int ra_attention_plain_mod(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
+                           const void* vcache, int act_dtype, const int* block_tables, int max_blocks,
+                           const int* token_list, const int* seq_of_token, const int* positions, int n_tokens,
+                           int block_size, int Hq, int Hkv, int d, float scale, int window, float softcap,
+                           const float* r1, const float* r2, hipStream_t stream);
+// act 2 of ra_act_mul with its bound: g <- min(g, lim), u <- clamp(u, -lim, lim), out = g sigmoid(1.702 g) (u + 1)
+int ra_act_mul_bounded(const void* gate_up, void* out, int act_dtype, int n_tokens, int intermediate, int group,
+                       int act, float lim, hipStream_t stream);
 
 int ra_gemm_plain(const void* A, const void* W, const void* bias, void* C, int in_dtype, int out_dtype,
                   int M, int N, int K, int lda, int ldc, hipStream_t stream);
@@ -119,6 +130,12 @@ int ra_attention_decode(const void* q, int q_stride, void* out, int out_stride, 
 // Where ra_attention_prefill_columns() is 2, bits 16-17 of the third may name the half of the heads a
 // workgroup computes (1 or 2; 0 or 3: all): the same tile listed twice, once with each, is computed by
 // two workgroups. A tile makes ra_attention_prefill_groups() workgroups.
+int ra_attention_decode_mod(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
+                            const void* vcache, const int* block_tables, int max_blocks,
+                            const int* token_list, const int* seq_of_token, const int* positions,
+                            int n_tokens, int block_size, int Hq, int Hkv, int d, float scale, int window,
+                            int chunk, int max_chunks, int waves, float* part_o, float* part_ml, float softcap,
+                            const float* r1, const float* r2, hipStream_t stream);
 int ra_attention_prefill_supports(int Hq, int Hkv, int d, int block_size);
 int ra_attention_prefill_tile(int Hq, int Hkv, int d);
 int ra_attention_prefill_columns(int Hq, int Hkv, int d);
@@ -137,6 +154,16 @@ int ra_attention_prefill_split(const void* q, int q_stride, void* out, int out_s
                                int n_tiles, const int* ranges, const int* merge_info, int n_merge, float* part_o,
                                float* part_ml, int block_size, int Hq, int Hkv, int d, float scale, int window,
                                hipStream_t stream);
+
+int ra_attention_prefill_mod(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
+                             const void* vcache, const int* block_tables, int max_blocks, const int* tile_info,
+                             int n_tiles, int block_size, int Hq, int Hkv, int d, float scale, int window,
+                             float softcap, const float* r1, const float* r2, hipStream_t stream);
+int ra_attention_prefill_split_mod(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
+                                   const void* vcache, const int* block_tables, int max_blocks, const int* tile_info,
+                                   int n_tiles, const int* ranges, const int* merge_info, int n_merge, float* part_o,
+                                   float* part_ml, int block_size, int Hq, int Hkv, int d, float scale, int window,
+                                   float softcap, const float* r1, const float* r2, hipStream_t stream);
 
 int ra_sample_slices(int vocab);
 int ra_sample(const float* logits, int n_rows, int vocab, int row_stride, const float* temperature,
@@ -259,6 +286,23 @@ int ra_moe_down_gated_chosen(const void* act, const void* w_down, const int* ids
                              int ldx, void* out, int act_dtype, int n_tokens, int top, int experts, int ff, int shared,
                              int width, hipStream_t stream);
 
+// ids[t, j] = table[token_ids[t], j] (table int32 [vocabulary, top]); weights[t, j] = 1 / top
+int ra_moe_table_route(const int* token_ids, const int* table, int top, int* ids, float* weights, int n_tokens,
+                       hipStream_t stream);
+
+// ---- sublayer.hip: the stream as an operand, results that enter behind a norm, norms over runs of columns, turns ----
+int ra_stream_cast(const float* x, void* out, int act_dtype, long n, hipStream_t stream);
+// y = sum_i scales[i] xs[i]; normed: y <- y / rms(y) * weight (weight_stride 1: a vector, 0: one number);
+// resid (float, or null) += y; copy (or null) = the new stream, or without resid the result, in copy_dtype
+int ra_sum_norm_add(const void* const* xs, const float* scales, int n, int in_dtype, const float* weight,
+                    int weight_stride, int normed, float eps, int n_tokens, int hidden, float* resid, void* copy,
+                    int copy_dtype, hipStream_t stream);
+int ra_span_rmsnorm(void* x, int act_dtype, long ld, int n_tokens, int n_spans, const int* col0, const int* width,
+                    const int* count, const float* const* w, float eps, hipStream_t stream);
+int ra_turn_heads(void* x, int act_dtype, long ld, int n_tokens, int heads, int head_stride, int width, int style,
+                  const int* positions, const float* inv_freq, float sign, const void* gate, long ldg, int gate_stride,
+                  hipStream_t stream);
+
 // C += acc_scale * (A . W^T) through the weight-streaming kernels (bfloat16 operands, float C; the limits of
 // ra_gemm_skinny / ra_gemm_wide with the accumulating epilogue)
 int ra_gemm_skinny_scaled(const void* A, const void* W, float* C, int M, int N, int K, int lda, int ldc,
@@ -267,7 +311,8 @@ int ra_gemm_wide_scaled(const void* A, const void* W, float* C, int M, int N, in
                         long scratch_floats, float acc_scale, hipStream_t stream);
 
 // ---- recurrent mixers (recurrent.hip) ----
-// floats of state a request slot holds for the scan kernels; kind 0: matrix memory, 1: delta rule; -1: sizes not taken
+// floats of state a request slot holds for the scan kernels; kind 0: matrix memory, 1: delta rule, 2: wkv, 3: a memory
+// fading by a constant a head; -1: sizes not taken
 long ra_scan_state_floats(int kind, int heads, int key_dim, int value_dim);
 // max_q_len: the most tokens a request brings (0: unknown; it only sizes the chunks that are staged)
 // gates [n_tokens, 2 heads] float pre-activations (input | forget); gates3 [n_tokens, 3 heads] scratch for the
@@ -296,6 +341,13 @@ int ra_wkv_scan(const void* proj, int act_dtype, int ld, int r_off, int k_off, i
                 const float* w0, const float* u, float* state, long slot_stride, const int* cu_tokens,
                 const int* state_slots, const int* fresh, int n_seqs, int n_tokens, int max_q_len, int heads, int dim,
                 float* out, hipStream_t stream);
+// kind 3 of ra_scan_state_floats. proj rows hold q, k (heads x key_dim each) and v (heads x value_dim) at the given
+// column offsets, before their silu (applied here, in float); decays float [heads]: S <- decays[h] S + k v^T, then
+// o = S^T q
+int ra_decay_scan(const void* proj, int act_dtype, int ld, int q_off, int k_off, int v_off, const float* decays,
+                  float* state, long slot_stride, const int* cu_tokens, const int* state_slots, const int* fresh,
+                  int n_seqs, int n_tokens, int max_q_len, int heads, int key_dim, int value_dim, float* out,
+                  hipStream_t stream);
 int ra_head_norm_gate(const float* read, const float* weight, int per_head_weight, const void* gate, int ldg,
                       int act_dtype, int silu, float eps, int n_tokens, int heads, int value_dim, void* out,
                       hipStream_t stream);

@@ -15,7 +15,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library links against)
 
 from ..csrc import build as _build
 
-ABI_VERSION = 22
+ABI_VERSION = 23
 
 
 class KernelLibraryError(RuntimeError):
@@ -77,6 +77,17 @@ _SIGNATURES = {
     "ra_delta_rule_scan": [P, I, P, P, P, P, c_long, P, P, P, I, I, I, I, I, I, I, P, P],
     "ra_head_norm_gate": [P, P, I, P, I, I, I, F, I, I, I, P, P],
     "ra_normed_mean": [P, P, I, I, F, I, I, P, P, F, P],
+    "ra_attention_plain_mod": [P, I, P, I, P, P, I, P, I, P, P, P, I, I, I, I, I, F, I, F, P, P, P],
+    "ra_attention_decode_mod": [P, I, P, I, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, I, P, P, F, P, P, P],
+    "ra_attention_prefill_mod": [P, I, P, I, P, P, P, I, P, I, I, I, I, I, F, I, F, P, P, P],
+    "ra_attention_prefill_split_mod": [P, I, P, I, P, P, P, I, P, I, P, P, I, P, P, I, I, I, I, F, I, F, P, P, P],
+    "ra_act_mul_bounded": [P, P, I, I, I, I, I, F, P],
+    "ra_decay_scan": [P, I, I, I, I, I, P, P, c_long, P, P, P, I, I, I, I, I, I, P, P],
+    "ra_moe_table_route": [P, P, I, P, P, I, P],
+    "ra_stream_cast": [P, P, I, c_long, P],
+    "ra_sum_norm_add": [P, P, I, I, P, I, I, F, I, I, P, P, I, P],
+    "ra_span_rmsnorm": [P, I, c_long, I, I, P, P, P, P, F, P],
+    "ra_turn_heads": [P, I, c_long, I, I, I, I, I, P, P, F, P, c_long, I, P],
     "ra_stream_read": [P, c_long, P, P],
     "ra_mfma_loop": [I, I, I, P, P, P],
 }

@@ -194,10 +194,12 @@ class HipKernels:
                      int(rotary_dim), int(rope_style), slots.data_ptr(), kcache.data_ptr(), vcache.data_ptr(),
                      kcache.shape[2] * 16, T, num_heads, num_kv_heads, head_dim, _stream())
 
-    GATE_ACTS = {"silu": 0, "gelu_tanh": 1}
+    GATE_ACTS = {"silu": 0, "gelu_tanh": 1, "swish_bounded": 2}
 
-    def silu_mul(self, gate_up: torch.Tensor, out: torch.Tensor, group: int = 0, act: str = "silu") -> None:
-        """out = act(gate) * up, act "silu" or "gelu_tanh" (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))).
+    def silu_mul(self, gate_up: torch.Tensor, out: torch.Tensor, group: int = 0, act: str = "silu",
+                 limit: float = 0.0) -> None:
+        """out = act(gate) * up, act "silu" or "gelu_tanh" (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))), or
+        "swish_bounded": g <- min(gate, limit), u <- clamp(up, -limit, limit), out = g sigmoid(1.702 g) (u + 1).
         ``group`` 0: gate_up is [gate | up]; ``group`` g > 0: runs of g gate columns and g up columns alternate."""
         _dev(gate_up, out)
         T, I = out.shape
@@ -208,8 +210,10 @@ class HipKernels:
             raise ValueError(f"silu_mul: width {I} is not a whole number of runs of {group}")
         if act not in self.GATE_ACTS:
             raise ValueError(f"silu_mul: activation {act!r}; built: {sorted(self.GATE_ACTS)}")
-        library.call("ra_act_mul", gate_up.data_ptr(), out.data_ptr(), _tag(out, "silu_mul"), T, I,
-                     int(group), self.GATE_ACTS[act], _stream())
+        if act == "swish_bounded" and not limit > 0.0:
+            raise ValueError("silu_mul: the bounded activation needs a positive limit")
+        library.call("ra_act_mul_bounded", gate_up.data_ptr(), out.data_ptr(), _tag(out, "silu_mul"), T, I,
+                     int(group), self.GATE_ACTS[act], float(limit), _stream())
 
     # ------------------------------------------------------------- attention
     SHORT_PORTION = 4     # portions up to this many tokens go token by token through the decode kernel
@@ -217,8 +221,12 @@ class HipKernels:
 
     def attention(self, q: torch.Tensor, q_stride: int, out: torch.Tensor, kcache: torch.Tensor,
                   vcache: torch.Tensor, batch, num_heads: int, num_kv_heads: int, head_dim: int,
-                  scale: float, window: int, group: int) -> None:
+                  scale: float, window: int, group: int, softcap: float = 0.0, distance=None) -> None:
         """Attention of every token of the step over its request's cache.
+
+        ``softcap`` > 0: score <- softcap * tanh(score / softcap); ``distance`` = (r1, r2), two float32 vectors
+        with one entry a query head: score <- score - r1[h] * ln(1 + r2[h] * (query position - key position)),
+        behind the cap. Every kernel below applies them alike.
 
         ``q`` is the buffer whose row ``t`` holds the query heads of token t at
         its start (row stride ``q_stride`` elements); ``batch`` is the step's
@@ -229,9 +237,10 @@ class HipKernels:
         float32, go to the plain kernel.
         """
         lib = library.load()
+        mod = self._score_mod(softcap, distance, num_heads, q.device)
         if q.dtype != torch.bfloat16:
             return self.attention_plain(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
-                                        head_dim, scale, window, group)
+                                        head_dim, scale, window, group, mod=mod)
         bs = kcache.shape[2] * 16
         tile = lib.ra_attention_prefill_tile(num_heads, num_kv_heads, head_dim)
         # query tiles that give every CU one workgroup
@@ -256,26 +265,39 @@ class HipKernels:
             with torch.cuda.stream(side):           # its scratch comes from, and goes back to, the side stream's pool
                 self.attention_decode(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
                                       head_dim, scale, window, group, plan["decode_list"], plan["n_decode"],
-                                      plan["decode_max_ctx"])
+                                      plan["decode_max_ctx"], mod=mod)
         elif plan["n_decode"]:
             if dec_ok:
                 self.attention_decode(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
                                       head_dim, scale, window, group, plan["decode_list"], plan["n_decode"],
-                                      plan["decode_max_ctx"])
+                                      plan["decode_max_ctx"], mod=mod)
             else:
                 self.attention_plain(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
-                                     head_dim, scale, window, group, plan["decode_list"], plan["n_decode"])
+                                     head_dim, scale, window, group, plan["decode_list"], plan["n_decode"], mod=mod)
         if plan["n_tiles"]:
             if pre_ok:
                 self.attention_prefill(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
                                        head_dim, scale, window, group, plan["tiles"], plan["n_tiles"],
                                        plan.get("ranges"), plan.get("merge"), plan.get("n_merge", 0),
-                                       plan.get("n_slots", 0))
+                                       plan.get("n_slots", 0), mod=mod)
             else:
                 self.attention_plain(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
-                                     head_dim, scale, window, group, plan["prefill_list"], plan["n_prefill"])
+                                     head_dim, scale, window, group, plan["prefill_list"], plan["n_prefill"], mod=mod)
         if side is not None:
             torch.cuda.current_stream().wait_stream(side)
+
+    @staticmethod
+    def _score_mod(softcap: float, distance, num_heads: int, device):
+        """(softcap, r1 pointer or None, r2 pointer or None) for the kernels' ``_mod`` entry points, checked."""
+        if softcap < 0.0:
+            raise ValueError("attention: a negative score cap")
+        if distance is None:
+            return (float(softcap), None, None)
+        r1, r2 = distance
+        for r in (r1, r2):
+            if r.dtype != torch.float32 or r.shape != (num_heads,) or not r.is_contiguous() or r.device != device:
+                raise ValueError(f"attention: the distance term takes two float32 vectors of {num_heads} entries")
+        return (float(softcap), r1.data_ptr(), r2.data_ptr())
 
     def shared_head_limit(self, head_dim: int, block_size: int = 16) -> int:
         """Query heads that may share one KV head in a call of :meth:`attention` and still take the
@@ -493,15 +515,15 @@ class HipKernels:
         return tables
 
     def attention_plain(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim,
-                        scale, window, group, token_list=None, n_listed=None) -> None:
+                        scale, window, group, token_list=None, n_listed=None, mod=(0.0, None, None)) -> None:
         tables = self._check_attention(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
                                        head_dim, group)
         n = batch.num_tokens if token_list is None else int(n_listed)
-        library.call("ra_attention_plain", q.data_ptr(), q_stride, out.data_ptr(), out.stride(0),
+        library.call("ra_attention_plain_mod", q.data_ptr(), q_stride, out.data_ptr(), out.stride(0),
                      kcache.data_ptr(), vcache.data_ptr(), _tag(q, "attention"), tables.data_ptr(),
                      tables.shape[1], _ptr(token_list), batch.seq_of_token.data_ptr(),
                      batch.positions.data_ptr(), n, kcache.shape[2] * 16, num_heads, num_kv_heads, head_dim,
-                     float(scale), int(window), _stream())
+                     float(scale), int(window), mod[0], mod[1], mod[2], _stream())
 
     # The decode kernel runs in workgroups of 12 waves from this many (token, KV head) pairs on, or over
     # contexts longer than this; below both, in workgroups of 4 (measured with 32 query heads over 8 KV
@@ -558,7 +580,7 @@ class HipKernels:
 
     def attention_decode(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim,
                          scale, window, group, token_list=None, n_listed=None, max_ctx=None,
-                         chunk=None, waves=None) -> None:
+                         chunk=None, waves=None, mod=(0.0, None, None)) -> None:
         tables = self._check_attention(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
                                        head_dim, group)
         if q.dtype != torch.bfloat16:
@@ -578,15 +600,16 @@ class HipKernels:
             part_ml = torch.empty((pairs, max_chunks, G, 2), dtype=torch.float32, device=q.device)
         # every request of the step brings one token: token t is request t, and the kernel need not look it up
         one_each = token_list is None and batch.num_tokens == batch.num_seqs
-        library.call("ra_attention_decode", q.data_ptr(), q_stride, out.data_ptr(), out.stride(0),
+        library.call("ra_attention_decode_mod", q.data_ptr(), q_stride, out.data_ptr(), out.stride(0),
                      kcache.data_ptr(), vcache.data_ptr(), tables.data_ptr(), tables.shape[1],
                      _ptr(token_list), None if one_each else batch.seq_of_token.data_ptr(), batch.positions.data_ptr(), n,
                      kcache.shape[2] * 16, num_heads, num_kv_heads, head_dim, float(scale), int(window),
-                     int(chunk), int(max_chunks), int(waves), _ptr(part_o), _ptr(part_ml), _stream())
+                     int(chunk), int(max_chunks), int(waves), _ptr(part_o), _ptr(part_ml), mod[0], mod[1], mod[2],
+                     _stream())
 
     def attention_prefill(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim,
                           scale, window, group, tiles, n_tiles, ranges=None, merge=None, n_merge: int = 0,
-                          n_slots: int = 0) -> None:
+                          n_slots: int = 0, mod=(0.0, None, None)) -> None:
         """``tiles``: four ints a listed query tile (request row, first token row, queries, first
         position). With ``ranges`` (three ints a listed tile: first key, one past the last, the part's
         slot or -1) some tiles are listed in several parts by keys, and ``merge`` (four ints a cut tile:
@@ -606,16 +629,16 @@ class HipKernels:
                                  dtype=torch.float32, device=q.device)
             part_ml = torch.empty(int(lib.ra_attention_prefill_part_floats(num_heads, num_kv_heads, head_dim, n_slots, 1)),
                                   dtype=torch.float32, device=q.device)
-            library.call("ra_attention_prefill_split", q.data_ptr(), q_stride, out.data_ptr(), out.stride(0),
+            library.call("ra_attention_prefill_split_mod", q.data_ptr(), q_stride, out.data_ptr(), out.stride(0),
                          kcache.data_ptr(), vcache.data_ptr(), tables.data_ptr(), tables.shape[1],
                          tiles.data_ptr(), int(n_tiles), ranges.data_ptr(), merge.data_ptr(), int(n_merge),
                          part_o.data_ptr(), part_ml.data_ptr(), kcache.shape[2] * 16, num_heads, num_kv_heads,
-                         head_dim, float(scale), int(window), _stream())
+                         head_dim, float(scale), int(window), mod[0], mod[1], mod[2], _stream())
             return
-        library.call("ra_attention_prefill", q.data_ptr(), q_stride, out.data_ptr(), out.stride(0),
+        library.call("ra_attention_prefill_mod", q.data_ptr(), q_stride, out.data_ptr(), out.stride(0),
                      kcache.data_ptr(), vcache.data_ptr(), tables.data_ptr(), tables.shape[1],
                      tiles.data_ptr(), int(n_tiles), kcache.shape[2] * 16, num_heads, num_kv_heads, head_dim,
-                     float(scale), int(window), _stream())
+                     float(scale), int(window), mod[0], mod[1], mod[2], _stream())
 
     # ---------------------------------------------------------------- linear
     def linear(self, x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor,
@@ -1000,7 +1023,7 @@ class HipKernels:
                      1 if gate_per_head else 0, _tag(x, "head_linear"), T, H, N, K, _stream())
 
     # ------------------------------------------------------ recurrent mixers
-    _SCAN_KINDS = {"matrix_memory": 0, "delta_rule": 1, "wkv": 2}
+    _SCAN_KINDS = {"matrix_memory": 0, "delta_rule": 1, "wkv": 2, "decay_memory": 3}
 
     def scan_state_floats(self, kind: str, heads: int, key_dim: int, value_dim: int) -> int:
         """Floats of a request's state slot that the scan kernel of ``kind`` ("matrix_memory", "delta_rule", "wkv")
@@ -1205,6 +1228,113 @@ class HipKernels:
         library.call("ra_head_norm_gate", read.data_ptr(), weight.data_ptr(), 1 if per_head else 0, gate.data_ptr(),
                      gate.stride(0), _tag(out, "head_norm_gate"), 1 if kind == "silu" else 0, float(eps), T, int(heads),
                      int(value_dim), out.data_ptr(), _stream())
+
+    # ------------------------------------------------ sublayers that read the stream, results behind a norm
+    def stream_cast(self, resid: torch.Tensor, out: torch.Tensor) -> None:
+        """out = resid in the activations' type: the float stream as a product's operand."""
+        _dev(resid, out)
+        if resid.dtype != torch.float32 or not resid.is_contiguous() or out.shape != resid.shape or not out.is_contiguous():
+            raise ValueError("stream_cast: a contiguous float32 stream and a contiguous copy of its shape")
+        library.call("ra_stream_cast", resid.data_ptr(), out.data_ptr(), _tag(out, "stream_cast"), resid.numel(), _stream())
+
+    def sum_norm_add(self, xs, scales, weight: Optional[torch.Tensor], eps: float,
+                     resid: Optional[torch.Tensor] = None, copy: Optional[torch.Tensor] = None) -> None:
+        """y = sum_i scales[i] * xs[i] row by row in float; with ``weight`` (float32, [width] or one number)
+        y <- y / rms(y) * weight; ``resid += y`` where the float stream is given; ``copy`` (any of the two
+        types) gets the new stream, or without ``resid`` the result."""
+        import ctypes
+        n = len(xs)
+        if not 1 <= n <= 4 or len(scales) != n:
+            raise ValueError(f"sum_norm_add: {n} inputs with {len(scales)} factors (1 to 4 of each)")
+        _dev(*xs, weight, resid, copy)
+        T, h = xs[0].shape
+        for x in xs:
+            if x.shape != (T, h) or x.dtype != xs[0].dtype or not x.is_contiguous():
+                raise ValueError("sum_norm_add: the inputs are contiguous [T, width] of one dtype")
+        if weight is not None and (weight.dtype != torch.float32 or weight.numel() not in (1, h) or not weight.is_contiguous()):
+            raise ValueError(f"sum_norm_add: the weight is float32, one number or [{h}]")
+        if resid is None and copy is None:
+            raise ValueError("sum_norm_add: the result goes into the stream or into a copy")
+        for name, t, dt in (("resid", resid, torch.float32), ("copy", copy, None)):
+            if t is not None and (t.shape != (T, h) or not t.is_contiguous() or (dt is not None and t.dtype != dt)):
+                raise ValueError(f"sum_norm_add: {name} is contiguous [T, width]")
+        px = (ctypes.c_void_p * n)(*[x.data_ptr() for x in xs])
+        ps = (ctypes.c_float * n)(*[float(v) for v in scales])
+        library.call("ra_sum_norm_add", px, ps, n, _tag(xs[0], "sum_norm_add"), _ptr(weight),
+                     0 if weight is None or weight.numel() == 1 else 1, 0 if weight is None else 1, float(eps), T, h,
+                     _ptr(resid), _ptr(copy), _tag(copy, "sum_norm_add copy") if copy is not None else 0, _stream())
+
+    def span_rmsnorm(self, x: torch.Tensor, spans, eps: float) -> None:
+        """Runs of columns of every row of ``x``, in place: ``spans`` = up to two (first column, width, weight
+        float32 [width], count); a run is divided by sqrt(sum of squares / count + eps) and multiplied by its weight."""
+        import ctypes
+        n = len(spans)
+        if not 1 <= n <= 2:
+            raise ValueError("span_rmsnorm: one or two runs")
+        _dev(x, *[s[2] for s in spans])
+        if x.dim() != 2 or x.stride(1) != 1:
+            raise ValueError("span_rmsnorm: rows with contiguous columns")
+        for c0, w, wt, cnt in spans:
+            if wt.dtype != torch.float32 or wt.shape != (w,) or not wt.is_contiguous() or c0 < 0 or c0 + w > x.shape[1] or cnt <= 0:
+                raise ValueError(f"span_rmsnorm: run at {c0} of {w} with weight {tuple(wt.shape)} {wt.dtype}")
+        ints = lambda k: (ctypes.c_int * n)(*[int(s[k]) for s in spans])
+        pw = (ctypes.c_void_p * n)(*[s[2].data_ptr() for s in spans])
+        library.call("ra_span_rmsnorm", x.data_ptr(), _tag(x, "span_rmsnorm"), x.stride(0), x.shape[0], n, ints(0),
+                     ints(1), ints(3), pw, float(eps), _stream())
+
+    def turn_heads(self, x: torch.Tensor, heads: int, head_stride: int, width: int, style: int,
+                   positions: Optional[torch.Tensor], inv_freq: Optional[torch.Tensor], sign: float = 1.0,
+                   gate: Optional[torch.Tensor] = None, gate_stride: int = 0) -> None:
+        """In place on ``x`` (rows of ``heads`` heads ``head_stride`` apart; a column range of a wider buffer
+        will do): the first ``width`` entries of every head turn by sign * position, pair m being (m, m + width / 2)
+        (``style`` 0) or (2m, 2m + 1) (1), by position * inv_freq[m]; with ``gate`` (heads ``gate_stride`` apart)
+        every entry of a head is then multiplied by the sigmoid of the gate's entry at the same place."""
+        _dev(x, positions, inv_freq, gate)
+        T = x.shape[0]
+        if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] < heads * head_stride:
+            raise ValueError(f"turn_heads: rows of {heads} heads of {head_stride}")
+        if width:
+            _int32(positions, "positions", T)
+            if inv_freq.dtype != torch.float32 or inv_freq.numel() < width // 2 or not inv_freq.is_contiguous():
+                raise ValueError("turn_heads: inv_freq is float32 with width / 2 entries")
+        if gate is not None and (gate.dim() != 2 or gate.shape[0] != T or gate.stride(1) != 1 or gate.dtype != x.dtype
+                                 or gate.shape[1] < (heads - 1) * gate_stride + head_stride):
+            raise ValueError("turn_heads: the gate's rows do not cover the heads")
+        library.call("ra_turn_heads", x.data_ptr(), _tag(x, "turn_heads"), x.stride(0), T, int(heads), int(head_stride),
+                     int(width), int(style), _ptr(positions), _ptr(inv_freq), float(sign), _ptr(gate),
+                     gate.stride(0) if gate is not None else 0, int(gate_stride), _stream())
+
+    def decay_scan(self, proj: torch.Tensor, q_off: int, k_off: int, v_off: int, decays: torch.Tensor,
+                   state: torch.Tensor, batch, heads: int, key_dim: int, value_dim: int, out: torch.Tensor) -> None:
+        """S <- decays[h] S + k v^T, o = S^T q head by head and token by token, q, k and v being the silu of
+        ``proj``'s columns at the given offsets; the state [slots, floats] is float32, ``out`` float32
+        [T, heads * value_dim]."""
+        _dev(proj, decays, state, out)
+        T = proj.shape[0]
+        self._check_scan("decay_scan", state, batch, T)
+        if decays.dtype != torch.float32 or decays.shape != (heads,) or not decays.is_contiguous():
+            raise ValueError(f"decay_scan: one float32 factor a head ({heads})")
+        if proj.dim() != 2 or proj.stride(1) != 1 or max(q_off, k_off) + heads * key_dim > proj.shape[1] \
+                or v_off + heads * value_dim > proj.shape[1]:
+            raise ValueError("decay_scan: the projection rows do not hold q, k and v at the given offsets")
+        if out.shape != (T, heads * value_dim) or out.dtype != torch.float32 or not out.is_contiguous():
+            raise ValueError(f"decay_scan: out is contiguous float32 [T, {heads * value_dim}]")
+        library.call("ra_decay_scan", proj.data_ptr(), _tag(proj, "decay_scan"), proj.stride(0), int(q_off), int(k_off),
+                     int(v_off), decays.data_ptr(), state.data_ptr(), state.stride(0), batch.cu_tokens.data_ptr(),
+                     batch.state_slots.data_ptr(), batch.fresh.data_ptr(), batch.num_seqs, T, int(batch.max_q_len),
+                     int(heads), int(key_dim), int(value_dim), out.data_ptr(), _stream())
+
+    def moe_table_route(self, token_ids: torch.Tensor, table: torch.Tensor, ids: torch.Tensor,
+                        weights: torch.Tensor) -> None:
+        """ids[t, j] = table[token_ids[t], j], weights[t, j] = 1 / top: experts looked up by token id."""
+        _dev(token_ids, table, ids, weights)
+        T, top = ids.shape
+        _int32(token_ids, "token ids", T)
+        if table.dtype != torch.int32 or table.dim() != 2 or table.shape[1] != top or not table.is_contiguous():
+            raise ValueError(f"moe_table_route: an int32 table [vocabulary, {top}]")
+        self._check_choice("moe_table_route", ids, weights, T, top)
+        library.call("ra_moe_table_route", token_ids.data_ptr(), table.data_ptr(), top, ids.data_ptr(),
+                     weights.data_ptr(), T, _stream())
 
     def normed_mean(self, xs, weights, eps: float, out: Optional[torch.Tensor] = None,
                     resid: Optional[torch.Tensor] = None, scale: float = 1.0) -> None:

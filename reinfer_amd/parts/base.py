@@ -138,6 +138,23 @@ class NormTarget:
         return self.norm.weight, self.x, self.norm.eps
 
 
+@dataclass
+class StreamCopy:
+    """What a block hands on in place of a pending addend when everything is in the stream already and it also
+    holds the stream in the activations' type (``x`` [T, width]): a block whose parts read the stream itself takes
+    it as their operand; any other block treats it as "nothing pending"."""
+    x: torch.Tensor
+
+
+@dataclass
+class ScaledTerms:
+    """A part's result left as a sum to be formed, sum_i scales[i] * terms[i] ([T, width] tensors of one dtype):
+    handed back by a part that declares ``returns_terms`` to a caller that asked with ``terms_ok=True`` and adds
+    the terms up itself, in float, in the kernel that consumes the sum."""
+    terms: list
+    scales: list
+
+
 def split_input(x):
     """(tensor, row sums or None) of a part's input, plain or :class:`RowScaled`."""
     if isinstance(x, RowScaled):

@@ -1,5 +1,8 @@
 """How norm, mixer and feed-forward are arranged in a layer.
 
+"outnorm": x += norm1(mixer(x)); x += norm2(ffn(x)): the parts read the stream itself and the norm stands on
+each part's result alone (a layer may have no feed-forward).
+
 "prenorm": x += mixer(norm(x)); x += ffn(norm(x))
 (crates/cuda/src/engine.rs:4075-4314); with ``residual_scale`` s both addends enter times s, and a layer
 may have no feed-forward (then it has no second norm either). The residual stream is float. A block
@@ -16,7 +19,7 @@ import torch
 
 from ..config.schema import BlockSpec
 from ..weights import VECTOR, ParamDecl
-from .base import JointNeed, LayerCache, StateNeed
+from .base import JointNeed, LayerCache, ScaledTerms, StateNeed, StreamCopy
 from .registry import lookup, register_block
 
 
@@ -259,3 +262,99 @@ class ParallelBlock:
         for a in addends[:-1]:
             kernels.current().stream_add(resid, a)
         return addends[-1] if addends else None
+
+
+@register_block("outnorm")
+class OutNormBlock:
+    """x <- x + norm1(mixer(x)); x <- x + norm2(ffn(x)): both parts read the residual stream itself (in the
+    activations' type for their products), and each result is normed before it enters. The stream and the norms
+    are float. One kernel forms the part's result (a sum of scaled terms where the mixer hands back several),
+    norms it, adds it into the stream and writes the new stream in the activations' type for the part that reads
+    it next; the last copy is handed on to the next block (:class:`StreamCopy`). A block without a feed-forward
+    (``spec.ffn`` None) has no second norm."""
+
+    @classmethod
+    def declare_params(cls, spec: BlockSpec) -> List[ParamDecl]:
+        p = spec.prefix
+        out = lookup("norm", spec.mixer_norm.kind).declare_params(spec.mixer_norm, p + spec.mixer_norm_name)
+        out += lookup("mixer", spec.mixer.kind).declare_params(spec.mixer, p + spec.mixer_prefix)
+        if spec.ffn is not None:
+            out += lookup("norm", spec.ffn_norm.kind).declare_params(spec.ffn_norm, p + spec.ffn_norm_name)
+            out += lookup("feed_forward", spec.ffn.kind).declare_params(spec.ffn, p + spec.ffn_prefix)
+        return out
+
+    def __init__(self, spec: BlockSpec, weights: Dict[str, torch.Tensor], dtype: torch.dtype,
+                 device: torch.device):
+        missing = [n for n in ("mixer", "mixer_norm") if getattr(spec, n) is None]
+        if spec.ffn is not None and spec.ffn_norm is None:
+            missing.append("ffn_norm")
+        if missing:
+            raise ValueError(f"an outnorm block is made of a mixer with a norm behind it and at most a feed-forward "
+                             f"with a norm behind it; block {spec.prefix!r} names no {', '.join(missing)}")
+        p = spec.prefix
+        self.spec, self.dtype = spec, dtype
+        self.mixer_norm = lookup("norm", spec.mixer_norm.kind)(spec.mixer_norm, weights, p + spec.mixer_norm_name,
+                                                               dtype, device)
+        self.mixer = lookup("mixer", spec.mixer.kind)(spec.mixer, weights, p + spec.mixer_prefix, dtype, device)
+        self.ffn_norm = self.ffn = None
+        if spec.ffn is not None:
+            self.ffn_norm = lookup("norm", spec.ffn_norm.kind)(spec.ffn_norm, weights, p + spec.ffn_norm_name,
+                                                               dtype, device)
+            self.ffn = lookup("feed_forward", spec.ffn.kind)(spec.ffn, weights, p + spec.ffn_prefix, dtype, device)
+        for n in (self.mixer_norm, self.ffn_norm):
+            if n is not None and getattr(n, "groups", 1) != 1:
+                raise ValueError("an outnorm block norms a part's result over the whole width")
+
+    @property
+    def graph_safe(self) -> bool:
+        return bool(getattr(self.mixer, "graph_safe", False)
+                    and (self.ffn is None or getattr(self.ffn, "graph_safe", False)))
+
+    def cache_need(self):
+        return self.mixer.cache_need() if hasattr(self.mixer, "cache_need") else None
+
+    def parts(self):
+        return tuple(p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn) if p is not None)
+
+    @staticmethod
+    def _norm_weight(norm):
+        """The norm's weight as the kernel takes it: one float number, or a float vector over the width."""
+        w = getattr(norm, "scalar", None)
+        if w is None:
+            w = norm.weight if norm.weight.dtype == torch.float32 else norm.weight.float()
+        return w
+
+    def _enter(self, ops, resid, y, norm, want_copy: bool):
+        """resid += norm(y); -> the new stream in the activations' type (the stream itself where that is float)."""
+        if isinstance(y, ScaledTerms):
+            terms, scales = y.terms, y.scales
+        else:
+            terms, scales = [y], [1.0]
+        copy = None
+        if want_copy and self.dtype != torch.float32:
+            copy = torch.empty(resid.shape, dtype=self.dtype, device=resid.device)
+        ops.sum_norm_add(terms, scales, self._norm_weight(norm), norm.eps, resid=resid, copy=copy)
+        return copy if copy is not None else resid
+
+    def forward(self, resid: torch.Tensor, delta, batch, cache: Optional[LayerCache]):
+        from .. import kernels
+        ops = kernels.current()
+        if isinstance(delta, StreamCopy) and delta.x.dtype == self.dtype and delta.x.shape == resid.shape:
+            h = delta.x                       # the block before left the stream in the activations' type
+        else:
+            if isinstance(delta, torch.Tensor):
+                ops.stream_add(resid, delta)
+            if self.dtype == torch.float32:
+                h = resid
+            else:
+                h = torch.empty(resid.shape, dtype=self.dtype, device=resid.device)
+                ops.stream_cast(resid, h)
+        if getattr(self.mixer, "returns_terms", False):
+            a = self.mixer.forward(h, batch, cache, terms_ok=True)
+        else:
+            a = self.mixer.forward(h, batch, cache)
+        h = self._enter(ops, resid, a, self.mixer_norm, True)
+        if self.ffn is not None:
+            b = self.ffn.forward(h, batch)
+            h = self._enter(ops, resid, b, self.ffn_norm, True)
+        return StreamCopy(h) if h is not resid else None

@@ -6,8 +6,9 @@ their rows are interleaved in runs of 8 at load (8 gate rows, the 8 up rows of
 the same features, ...), so that for few tokens the product's epilogue applies
 the gate itself and for many the gate kernel reads both from one cache line.
 A width that is no multiple of 8 keeps [gate; up] and the separate gate kernel.
-The option ``act`` names another gate activation ("gelu_tanh": 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))));
-it is applied by the gate kernel behind the product.
+The option ``act`` names another gate activation ("gelu_tanh": 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)));
+"swish_bounded" with the option ``limit``: g <- min(gate, limit), u <- clamp(up, -limit, limit),
+g sigmoid(1.702 g) (u + 1)); it is applied by the gate kernel behind the product.
 """
 from __future__ import annotations
 
@@ -59,8 +60,11 @@ class SwiGLU:
             self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
         self.w_down = weights[prefix + dn]
         self.act = str(dict(spec.extra).get("act", "silu"))
-        if self.act not in ("silu", "gelu_tanh"):
-            raise ValueError(f"swiglu: gate activation {self.act!r}; built: silu, gelu_tanh")
+        if self.act not in ("silu", "gelu_tanh", "swish_bounded"):
+            raise ValueError(f"swiglu: gate activation {self.act!r}; built: silu, gelu_tanh, swish_bounded")
+        self.limit = float(dict(spec.extra).get("limit", 0.0))
+        if self.act == "swish_bounded" and not self.limit > 0.0:
+            raise ValueError("swiglu: the bounded activation needs a positive limit")
 
     def forward(self, x, batch, resid: Optional[torch.Tensor] = None, emit: Optional[NormTarget] = None,
                 resid_scale: float = 1.0):
@@ -76,7 +80,10 @@ class SwiGLU:
                 ops.linear(x, self.w_gate_up, gu)
             else:
                 ops.linear_skinny(x, self.w_gate_up, gu, row_sums=row_sums)
-            ops.silu_mul(gu, act, self.group, act=self.act)
+            if self.act == "swish_bounded":
+                ops.silu_mul(gu, act, self.group, act=self.act, limit=self.limit)
+            else:
+                ops.silu_mul(gu, act, self.group, act=self.act)
         elif self.group:
             if row_sums is None:
                 ops.gated_linear(x, self.w_gate_up, act)

@@ -28,6 +28,10 @@ its largest choice score); the weights are the chosen scores over their sum. The
 outputs stand for experts without matrices whose output is the token's input row; the shared expert's result is
 multiplied by the sigmoid of one more logit a token (its weight row lies behind the router's, so the same float
 product makes it). The experts' matrices and the two products are those of the second form.
+
+A fourth form (``activation`` "silu_gated", ``weights`` "table"): no router. An integer table [vocabulary, top]
+gives each token id its experts (the entries of a row differ), each weighing 1 / top; a kernel looks the step's
+token ids up, and everything behind the choice is the second form's.
 """
 from __future__ import annotations
 
@@ -37,7 +41,7 @@ import torch
 
 from .. import kernels
 from ..config.schema import FeedForwardSpec
-from ..weights import VECTOR, ParamDecl
+from ..weights import INT_TABLE, VECTOR, ParamDecl
 from .registry import register_feed_forward
 
 
@@ -57,7 +61,11 @@ class MixtureOfExperts:
                 out.append(ParamDecl(f"{prefix}e{e}.gate", (spec.intermediate, spec.hidden)))
             out += [ParamDecl(f"{prefix}e{e}.up", (spec.intermediate, spec.hidden)),
                     ParamDecl(f"{prefix}e{e}.down", (spec.hidden, spec.intermediate))]
-        out.append(ParamDecl(prefix + "router", (p.experts + p.identity, spec.hidden)))
+        if p.weights == "table":
+            out.append(ParamDecl(prefix + "table", (int(dict(spec.extra)["vocab"]), p.top), init=f"distinct:{p.experts}",
+                                 role=INT_TABLE))
+        else:
+            out.append(ParamDecl(prefix + "router", (p.experts + p.identity, spec.hidden)))
         if p.correction:
             out.append(ParamDecl(prefix + "correction", (p.experts + p.identity,), init="zeros", role=VECTOR))
         if p.shared:
@@ -75,7 +83,7 @@ class MixtureOfExperts:
         if p is None:
             raise ValueError("moe: the routing comes in FeedForwardSpec.params (MoESpec)")
         if (p.activation, p.weights) not in (("relu2", "softmax_chosen"), ("silu_gated", "sigmoid"),
-                                             ("silu_gated", "softmax")):
+                                             ("silu_gated", "softmax"), ("silu_gated", "table")):
             raise ValueError(f"moe: activation {p.activation!r} with weights {p.weights!r} is not built")
         self.spec = spec
         self.dtype = dtype
@@ -97,7 +105,14 @@ class MixtureOfExperts:
             raise ValueError("moe: a gate on the shared expert needs a shared expert")
         if (p.groups > 1 or p.shared) and not self.gated:
             raise ValueError("moe: groups of experts and a shared expert are built for the gated form")
-        self.router = weights[prefix + "router"]            # logits are accumulated and kept in float
+        self.table = None
+        if p.weights == "table":
+            if p.groups != 1 or p.top > p.experts:
+                raise ValueError(f"moe: a table of {p.top} choices among {p.experts} experts in {p.groups} groups")
+            self.table = weights[prefix + "table"].contiguous()
+            if int(self.table.min()) < 0 or int(self.table.max()) >= self.experts:
+                raise ValueError(f"moe: {prefix}table names experts outside 0..{self.experts - 1}")
+        self.router = weights[prefix + "router"] if self.table is None else None      # logits are accumulated and kept in float
         self.correction = weights[prefix + "correction"].float().contiguous() if p.correction else None
         if p.shared_gated:
             # the shared expert's gate is one more row of the float product that makes the router's logits
@@ -117,7 +132,7 @@ class MixtureOfExperts:
         self.w_up = torch.cat([weights[f"{prefix}e{e}.up"] for e in range(self.experts)], dim=0).contiguous()
         self.w_down = torch.cat([weights[f"{prefix}e{e}.down"] for e in range(self.experts)], dim=1).contiguous()
 
-    def _forward_gated(self, x, resid, resid_scale=1.0):
+    def _forward_gated(self, x, resid, resid_scale=1.0, batch=None):
         ops = kernels.current()
         p = self.routing
         T = x.shape[0]
@@ -126,7 +141,9 @@ class MixtureOfExperts:
         weights = torch.empty((T, self.top), dtype=torch.float32, device=x.device)
         routed = self.experts + self.identity
         shared_logit = None
-        if p.weights == "softmax":
+        if p.weights == "table":
+            ops.moe_table_route(batch.token_ids, self.table, ids, weights)
+        elif p.weights == "softmax":
             logits = ops.moe_route(x, self.router, self.top, ids, weights, scoring="softmax", groups=int(p.groups),
                                    groups_kept=int(p.groups_kept), correction=self.correction,
                                    norm_eps=float(p.norm_eps), outputs=routed)
@@ -171,7 +188,7 @@ class MixtureOfExperts:
 
     def forward(self, x, batch, resid: Optional[torch.Tensor] = None, resid_scale: float = 1.0):
         if self.gated:
-            return self._forward_gated(x, resid, resid_scale)
+            return self._forward_gated(x, resid, resid_scale, batch)
         if resid_scale != 1.0:
             resid = None                    # the ungated form adds its result as it is: the caller scales it
         ops = kernels.current()

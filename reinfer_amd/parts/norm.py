@@ -21,7 +21,8 @@ from .registry import register_norm
 class RMSNorm:
     @classmethod
     def declare_params(cls, spec: NormSpec, name: str) -> List[ParamDecl]:
-        return [ParamDecl(name, (spec.size,), init="norm", role=VECTOR)]
+        # a norm with one number for all coordinates stores a tensor without dimensions
+        return [ParamDecl(name, () if getattr(spec, "scalar", False) else (spec.size,), init="norm", role=VECTOR)]
 
     def __init__(self, spec: NormSpec, weights: Dict[str, torch.Tensor], name: str,
                  dtype: torch.dtype, device: torch.device):
@@ -31,6 +32,12 @@ class RMSNorm:
         if self.groups < 1 or spec.size % self.groups:
             raise ValueError(f"rmsnorm: width {spec.size} does not split into {self.groups} equal groups")
         self.weight = weights[name]
+        self.scalar = None
+        if getattr(spec, "scalar", False):
+            # one number: kept as a float tensor of one element for the kernels that take it so, and spread
+            # over the width for those that take a vector
+            self.scalar = weights[name].float().reshape(1).contiguous()
+            self.weight = self.scalar.expand(spec.size).contiguous()
         if spec.offset:
             # a weight stored around zero: the factor offset + w is made once, in float
             self.weight = (weights[name].float() + float(spec.offset)).contiguous()
@@ -53,6 +60,8 @@ class RMSNorm:
                 if scaled_ok:
                     return RowScaled(delta.x, delta.ss, self.eps, self.size)
             delta = None
+        elif delta is not None and not isinstance(delta, torch.Tensor):
+            delta = None                       # whatever else a block hands on: the sum is already in the stream
         n = resid.shape[0] if rows is None else rows.numel()
         out = torch.empty((n, self.size), dtype=self.dtype, device=resid.device)
         if self.groups != 1:

@@ -1,4 +1,5 @@
-"""Several mixers on one input, averaged: y = (1/n) sum_i rms(mixer_i(h)) * w_i.
+"""Several mixers on one input, averaged: y = (1/n) sum_i rms(mixer_i(h)) * w_i; or, with ``combine``
+"scaled_sum", added up with a constant each: y = sum_i s_i mixer_i(h), no norms and no weights.
 
 Each member reads the same normed input and keeps what it needs itself (keys and values in pages, a recurrent
 state in the request's slot); the layer's cache need is the members' needs side by side
@@ -14,7 +15,7 @@ import torch
 from .. import kernels
 from ..config.schema import MixerSpec
 from ..weights import VECTOR, ParamDecl
-from .base import JointNeed, LayerCache
+from .base import JointNeed, LayerCache, ScaledTerms
 from .registry import lookup, register_mixer
 
 
@@ -26,8 +27,9 @@ class SideBySide:
         out: List[ParamDecl] = []
         for sub, m in p.members:
             out += lookup("mixer", m.kind).declare_params(m, prefix + sub)
-        for sub, _ in p.members:
-            out.append(ParamDecl(prefix + sub + p.out_name, (spec.hidden,), init="norm", role=VECTOR))
+        if getattr(p, "combine", "normed_mean") == "normed_mean":
+            for sub, _ in p.members:
+                out.append(ParamDecl(prefix + sub + p.out_name, (spec.hidden,), init="norm", role=VECTOR))
         return out
 
     def __init__(self, spec: MixerSpec, weights: Dict[str, torch.Tensor], prefix: str, dtype: torch.dtype,
@@ -38,6 +40,16 @@ class SideBySide:
         self.spec, self.dtype = spec, dtype
         self.eps = float(p.norm_eps)
         self.members = [lookup("mixer", m.kind)(m, weights, prefix + sub, dtype, device) for sub, m in p.members]
+        self.combine = str(getattr(p, "combine", "normed_mean"))
+        if self.combine == "scaled_sum":
+            self.scales = [float(v) for v in p.scales]
+            if len(self.scales) != len(self.members):
+                raise ValueError(f"side_by_side: {len(self.scales)} factors for {len(self.members)} mixers")
+            self.adds_scaled = False
+            self.returns_terms = True      # forward(..., terms_ok=True) may hand back the addends with their factors
+            return
+        if self.combine != "normed_mean":
+            raise ValueError(f"side_by_side: combine {self.combine!r}; built: normed_mean, scaled_sum")
         self.out_weights = [weights[prefix + sub + p.out_name].float().contiguous() for sub, _ in p.members]
 
     @property
@@ -55,8 +67,15 @@ class SideBySide:
 
     adds_scaled = True      # forward(..., resid=, resid_scale=) adds the mean into the float stream itself
 
-    def forward(self, x, batch, cache: LayerCache, resid=None, resid_scale: float = 1.0):
+    def forward(self, x, batch, cache: LayerCache, resid=None, resid_scale: float = 1.0, terms_ok: bool = False):
         outs = [m.forward(x, batch, cache.members[i]) for i, m in enumerate(self.members)]
+        if self.combine == "scaled_sum":
+            if terms_ok:
+                # the caller adds the sum up itself (in the kernel that norms it and adds it to the stream)
+                return ScaledTerms(outs, list(self.scales))
+            out = torch.empty_like(outs[0])
+            kernels.current().sum_norm_add(outs, self.scales, None, 0.0, copy=out)
+            return out
         if resid is not None:
             kernels.current().normed_mean(outs, self.out_weights, self.eps, resid=resid, scale=resid_scale)
             return None

@@ -31,7 +31,7 @@ INT_TABLE = "int_table"
 class ParamDecl:
     name: str
     shape: Tuple[int, ...]
-    init: str = "normal"        # "normal": N(0, 0.02); "norm": U(0.8, 1.2); "zeros"; "int"
+    init: str = "normal"        # "normal": N(0, 0.02); "norm": U(0.8, 1.2); "zeros"; "int"; "distinct:m" (rows of different integers below m)
     role: str = MATRIX
     optional: bool = False      # absent is fine (e.g. a head that is tied)
 

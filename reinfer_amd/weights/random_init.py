@@ -93,6 +93,16 @@ def random_tensor(decl: ParamDecl, seed: int, dtype: torch.dtype,
         t = torch.zeros(decl.shape, dtype=torch.float32, device=device)
     elif decl.init == "int":
         t = torch.zeros(decl.shape, dtype=torch.int32, device=device)
+    elif decl.init.startswith("distinct:"):
+        # an integer table [rows, k] whose rows hold k different numbers below m ("distinct:m"): a hashed start
+        # a row, then its neighbours
+        m = int(decl.init.split(":", 1)[1])
+        rows, k = (int(v) for v in decl.shape)
+        if not 1 <= k <= m:
+            raise ValueError(f"{decl.name}: {k} different numbers below {m}")
+        i = torch.arange(rows, dtype=torch.int64, device=device)
+        start = (_mix(i * 2 + _signed(tensor_seed(seed, decl.name)) + _signed(0x9E3779B97F4A7C15)) >> 20) & 0x7FFFFFFF
+        t = ((start[:, None] + torch.arange(k, dtype=torch.int64, device=device)[None, :]) % m).to(torch.int32)
     else:
         raise ValueError(f"{decl.name}: unknown init {decl.init!r}")
     return t if decl.role == INT_TABLE else t.to(dtype)

@@ -165,7 +165,7 @@ class KernelDouble:
     # ---- recurrent mixers (state in a layout of this stand-in's own: the state is the kernels' private matter)
     @staticmethod
     def scan_state_floats(kind, heads, key_dim, value_dim):
-        return heads * key_dim * value_dim + (heads * (key_dim + 1) if kind == "matrix_memory" else 0)   # "delta_rule", "wkv": S alone
+        return heads * key_dim * value_dim + (heads * (key_dim + 1) if kind == "matrix_memory" else 0)   # the others: S alone
 
     @staticmethod
     def _requests(batch):
@@ -268,6 +268,65 @@ class KernelDouble:
                 kv = k[:, :, None] * v[:, None, :]
                 out[t] = torch.einsum("hkv,hk->hv", S + uu[:, :, None] * kv, r).reshape(-1)
                 S.mul_(w[t][:, :, None]).add_(kv)
+
+    def decay_scan(self, proj, q_off, k_off, v_off, decays, state, batch, H, dk, dv, out):
+        p = proj.float()
+        p = p * torch.sigmoid(p)
+        for first, rows, slot, fresh in self._requests(batch):
+            if slot < 0:
+                out[first:first + rows] = 0
+                continue
+            S = state[slot, :H * dk * dv].view(H, dk, dv)
+            if fresh:
+                S.zero_()
+            for t in range(first, first + rows):
+                q = p[t, q_off:q_off + H * dk].view(H, dk)
+                k = p[t, k_off:k_off + H * dk].view(H, dk)
+                v = p[t, v_off:v_off + H * dv].view(H, dv)
+                S.mul_(decays.float()[:, None, None]).add_(k[:, :, None] * v[:, None, :])
+                out[t] = torch.einsum("hkv,hk->hv", S, q).reshape(-1)
+
+    # ---- sublayers that read the stream, results behind a norm
+    def stream_cast(self, resid, out):
+        out.copy_(resid.to(out.dtype))
+
+    def sum_norm_add(self, xs, scales, weight, eps, resid=None, copy=None):
+        y = sum(float(s) * x.float() for x, s in zip(xs, scales))
+        if weight is not None:
+            y = y * torch.rsqrt((y * y).mean(-1, keepdim=True) + eps) * weight.float()
+        if resid is not None:
+            resid.add_(y)
+            y = resid
+        if copy is not None:
+            copy.copy_(y.to(copy.dtype))
+
+    def span_rmsnorm(self, x, spans, eps):
+        for c0, w, weight, count in spans:
+            v = x[:, c0:c0 + w].float()
+            v = v * torch.rsqrt((v * v).sum(-1, keepdim=True) / count + eps) * weight.float()
+            x[:, c0:c0 + w] = v.to(x.dtype)
+
+    def turn_heads(self, x, heads, head_stride, width, style, positions, inv_freq, sign=1.0, gate=None, gate_stride=0):
+        T = x.shape[0]
+        v = x[:, :heads * head_stride].float().reshape(T, heads, head_stride).clone()
+        if width:
+            half = width // 2
+            ang = sign * positions.float()[:, None] * inv_freq[:half].float()[None, :]
+            c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+            if style == 0:
+                a, b = v[..., :half].clone(), v[..., half:width].clone()
+                v[..., :half], v[..., half:width] = a * c - b * s, b * c + a * s
+            else:
+                a, b = v[..., 0:width:2].clone(), v[..., 1:width:2].clone()
+                v[..., 0:width:2], v[..., 1:width:2] = a * c - b * s, b * c + a * s
+        if gate is not None:
+            g = torch.stack([gate[:, h * gate_stride:h * gate_stride + head_stride].float() for h in range(heads)], dim=1)
+            v = v * torch.sigmoid(g)
+        x[:, :heads * head_stride] = v.reshape(T, heads * head_stride).to(x.dtype)
+
+    def moe_table_route(self, token_ids, table, ids, weights):
+        ids.copy_(table[token_ids.long()])
+        weights.fill_(1.0 / ids.shape[1])
 
     # ---- the token before, gated adds, row norms
     def token_shift(self, h, mu, state, keep_off, batch, out):
@@ -427,7 +486,7 @@ class KernelDouble:
 
     GATE_GROUP = 8
 
-    def silu_mul(self, gate_up, out, group=0, act="silu"):
+    def silu_mul(self, gate_up, out, group=0, act="silu", limit=0.0):
         T, I = out.shape
         if group:
             v = gate_up.view(T, I // group, 2, group).float()
@@ -436,6 +495,10 @@ class KernelDouble:
             g, u = gate_up[:, :I].float(), gate_up[:, I:].float()
         if act == "gelu_tanh":
             a = 0.5 * g * (1 + torch.tanh(0.7978845608028654 * (g + 0.044715 * g ** 3)))
+        elif act == "swish_bounded":
+            g = torch.clamp(g, max=limit)
+            a = g * torch.sigmoid(1.702 * g)
+            u = torch.clamp(u, min=-limit, max=limit) + 1.0
         else:
             a = g / (1 + torch.exp(-g))
         out.copy_((a * u).to(out.dtype))
@@ -486,7 +549,7 @@ class KernelDouble:
                 so[p] = sq[:, p * part:(p + 1) * part].sum(1)
 
     def attention(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim,
-                  scale, window, group):
+                  scale, window, group, softcap=0.0, distance=None):
         T = batch.num_tokens
         bs = kcache.shape[2] * 16
         kl, vl = unpack_k(kcache, head_dim), unpack_v(vcache, head_dim)      # [blocks, Hkv, bs, d]
@@ -503,6 +566,10 @@ class KernelDouble:
             V = vl[blk, :, keys % bs, :].float()
             for a in range(num_heads):
                 s = (K[:, a // ratio, :] @ qh[t, a]) * scale
+                if softcap > 0:
+                    s = softcap * torch.tanh(s / softcap)
+                if distance is not None:
+                    s = s - distance[0][a] * torch.log(1.0 + distance[1][a] * (p - keys).float())
                 pr = torch.softmax(s, dim=0)
                 out[t, a * head_dim:(a + 1) * head_dim] = (pr @ V[:, a // ratio, :]).to(out.dtype)
 
