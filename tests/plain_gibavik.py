@@ -61,7 +61,7 @@ def biased_attention(h, w, p, cfg, eps, shared=None, keep=None):
         for i in range(T):
             lo = max(0, i - window + 1) if window else 0
             dist = (i - torch.arange(lo, i + 1)).to(D)
-            s = (k[lo:i + 1, g] @ q[i, a]) * cfg["scale"] - r1 * torch.log(1.0 + r2 * dist)
+            s = (k[lo:i + 1, g] @ q[i, a]) * cfg.get("scale", dk ** -0.5) - r1 * torch.log(1.0 + r2 * dist)
             pr = torch.softmax(s, dim=0)
             out[i, a] = (pr[:, None] * v[lo:i + 1, g]).sum(0)
     return out.reshape(T, H * dv) @ w[p + "o"].T
@@ -105,7 +105,7 @@ def window_attention(h, w, p, cfg, eps):
         g = a // (H // G)
         for i in range(T):
             lo = max(0, i - window + 1) if window else 0
-            s = (k[lo:i + 1, g] @ q[i, a]) * cfg["scale"]
+            s = (k[lo:i + 1, g] @ q[i, a]) * cfg.get("scale", dk ** -0.5)
             if cap:
                 s = cap * torch.tanh(s / cap)
             out[i, a] = (torch.softmax(s, dim=0)[:, None] * v[lo:i + 1, g]).sum(0)
@@ -135,8 +135,8 @@ def decay_memory(h, w, p, cfg, eps):
 
 
 def parallel_mixers(h, w, p, cfg, eps):
-    return cfg["left_scale"] * window_attention(h, w, p + "left.", cfg["left"], eps) \
-        + cfg["right_scale"] * decay_memory(h, w, p + "right.", cfg["right"], eps)
+    return cfg.get("left_scale", 1.0) * window_attention(h, w, p + "left.", cfg["left"], eps) \
+        + cfg.get("right_scale", 1.0) * decay_memory(h, w, p + "right.", cfg["right"], eps)
 
 
 # ------------------------------------------------------------------ feed-forwards
