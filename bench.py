@@ -485,6 +485,61 @@ def detatar_sizes():
     return out
 
 
+# ---------------------------------------------------------------------------------------------------
+# --design gibavik: the Gibavik design beside the Kobolix design (the closest of the others: attention beside a
+# recurrent memory in one layer, gated experts, a scaled embedding) at equal size
+# ---------------------------------------------------------------------------------------------------
+def _gibavik_raw(width, vocab, pattern, attn, right, dense_ff, moe):
+    """``pattern``: a string of layer codes: A attention + dense, a attention + experts, p side-by-side + experts,
+    r attention on the keys of the attention layer before it + experts."""
+    heads, kv = attn
+    full = {"dim": 128, "heads": heads, "kv_heads": kv, "scale": 128 ** -0.5, "vdim": 128}
+    left = {"dim": 128, "heads": heads, "kv_heads": kv, "mask": {"size": 1024}, "rot": {"base": 1000000.0, "dims": 64},
+            "scale": 128 ** -0.5, "softcap": 30.0, "vdim": 128}
+    memory = {"decay": [1.0 - 2.0 ** -(2 + 6 * h / max(1, right - 1)) for h in range(right)], "dim": 128, "heads": right,
+              "vdim": 128}
+    pair = {"left": left, "left_scale": 0.6, "right": memory, "right_scale": 0.9}
+    dense = {"ff": dense_ff, "kind": "dense", "limit": 7.0}
+    experts = {"expert": {"ff": moe[2]}, "kind": "moe", "router": {"experts": moe[0], "top": moe[1]}}
+    layers = []
+    for c in pattern:
+        if c == "p":
+            layers.append({"type": "parallel", "mixer": pair, "mlp": experts})
+        elif c == "r":
+            j = max(i for i, L in enumerate(layers) if L["type"] == "attention" and "kv_from" not in L["mixer"])
+            layers.append({"type": "attention", "mixer": dict(full, kv_from=j), "mlp": experts})
+        else:
+            layers.append({"type": "attention", "mixer": full, "mlp": dense if c == "A" else experts})
+    return {"architecture": "Gibavik", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "embedding": {"scale": 12.0},
+            "logit_softcap": 15.0, "layers": layers}
+
+
+# (name, Gibavik configuration, its Kobolix twin, vocabulary, "kobolix"): as many layers, the same width, the same
+# attention heads and experts; a side-by-side layer (attention + delta rule) where Gibavik has one, and, where it has
+# an attention layer, a matrix-memory layer of as many heads (Kobolix has no layer of attention alone)
+def gibavik_sizes():
+    out = []
+    for name, width, attn, right, dense_ff, moe in (
+            ("w2048", 2048, (16, 4), 16, 5632, (16, 4, 512)),
+            ("w4096", 4096, (32, 8), 32, 11008, (16, 4, 1024))):
+        vocab, pattern = 32768, "Apapr"
+        raw = _gibavik_raw(width, vocab, pattern, attn, right, dense_ff, moe)
+        memory = {"dim": 128, "gate_cap": 15.0, "heads": attn[0], "vdim": 128}
+        pair = {"left": {"dim": 128, "heads": attn[0], "kv_heads": attn[1], "rot": {"base": 1000000.0, "dims": 64},
+                         "scale": 128 ** -0.5, "vdim": 128},
+                "right": {"conv": 4, "dim": 128, "heads": right, "kv_heads": right // 2, "vdim": 128}}
+        dense = {"ff": dense_ff, "kind": "dense"}
+        experts = {"expert": {"ff": moe[2]}, "kind": "moe",
+                   "router": {"experts": moe[0], "groups": {"count": 4, "keep": 2}, "scale": 2.5, "top": moe[1]}}
+        kinds = {"A": ("mlstm", memory, dense), "a": ("mlstm", memory, experts), "r": ("mlstm", memory, experts),
+                 "p": ("parallel", pair, experts)}
+        twin = {"architecture": "Kobolix", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.5,
+                "embedding": {"scale": 8.0},
+                "layers": [{"type": kinds[c][0], "mixer": kinds[c][1], "mlp": kinds[c][2]} for c in pattern]}
+        out.append((name, raw, twin, vocab, "kobolix"))
+    return out
+
+
 def design_run(args) -> int:
     """Prefill and decode throughput of the design (``--design``) and of its twin at each size, and the GPU time of a
     2,048-token prompt step and of a decode step at batch 8 by kernel class with each class's share of its
@@ -527,7 +582,8 @@ def design_run(args) -> int:
         return out
 
     results = {}
-    sizes = {"kobolix": kobolix_sizes, "puresun": design_sizes, "detatar": detatar_sizes}[args.design]()
+    sizes = {"kobolix": kobolix_sizes, "puresun": design_sizes, "detatar": detatar_sizes,
+             "gibavik": gibavik_sizes}[args.design]()
     twin_name = "qwen3"
     for name, p_raw, q_raw, vocab, *rest in sizes:
         twin_name = rest[0] if rest else "qwen3"
@@ -586,7 +642,7 @@ def main() -> int:
     ap.add_argument("--max-model-len", type=int, default=None, metavar="N",
                     help="context length (default: the shape's: 4096 at 8b, 8192 at 4b, 16384 at 32b)")
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes (default: the Qwen3-8B shape)")
-    ap.add_argument("--design", default=None, choices=["puresun", "kobolix", "detatar"],
+    ap.add_argument("--design", default=None, choices=["puresun", "kobolix", "detatar", "gibavik"],
                     help="instead of the default measurement: this design beside its closest other (the Qwen3 decoder; "
                          "for detatar, Puresun) at equal sizes")
     ap.add_argument("--size", default=None, help="with --design: this size alone (w2048 or w4096)")

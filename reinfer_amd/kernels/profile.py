@@ -38,7 +38,10 @@ _OTHER = {"latent_prep": "latent norm + rotation + cache write", "head_linear": 
           "delta_rule_scan": "delta rule scan", "head_norm_gate": "head norm + gate",
           "normed_mean": "mean of normed mixers", "moe_silu_gate_scale": "expert activation",
           "wkv_scan": "wkv scan", "token_shift": "mix with the row before", "gated_stream_add": "gated stream add",
-          "rows_rmsnorm": "row norm", "tanh_rows": "tanh", "moe_identity_add": "identity experts"}
+          "rows_rmsnorm": "row norm", "tanh_rows": "tanh", "moe_identity_add": "identity experts",
+          "stream_cast": "stream as operand", "sum_norm_add": "sum + norm + stream add",
+          "span_rmsnorm": "projection norm", "turn_heads": "turn of heads (+ gate)", "decay_scan": "decay scan",
+          "moe_table_route": "router"}
 
 
 class TimedKernels:

@@ -285,3 +285,49 @@ def test_trace_run_kobolix(tmp_path, which, dtype):
         assert o == rows.shape[0]
     for r in seqs:
         assert_close(torch.cat(got[r]), refs[r], dtype, r)
+
+
+@pytest.mark.parametrize("which,dtype", [("A", "float32"), ("C", "bfloat16"), ("B", "float32")])
+def test_trace_run_gibavik(tmp_path, which, dtype):
+    """A design with windows of several sizes, a layer that reads another layer's keys and memories in state slots
+    through the same program: five requests on four state slots and a cache for the 320 tokens that the four live
+    ones hold at most, portions beside single tokens, a request left out of a step, slots and blocks taken again."""
+    import gibavik_helpers as gh
+    import plain_gibavik
+    from test_gibavik_engine import assert_close
+    folder = gh.make_folder(tmp_path, which, dtype)
+    raw, weights = gh.read_folder(folder)
+    V = raw["vocab"]
+    lens = {"a": 70, "b": 41, "c": 50, "d": 9, "e": 30}
+    seqs = {r: random_tokens(n, V, 10 + i) for i, (r, n) in enumerate(lens.items())}
+    refs = {r: plain_gibavik.forward(raw, weights, t).float() for r, t in seqs.items()}
+    plan = [[("a", 33), ("b", 2)], [("a", 36), ("c", 17), ("d", 3)], [("b", 38), ("d", 1), ("c", 2)],
+            [("a", 1), ("b", 1), ("c", 30), ("d", 5)], [("c", 1), ("e", 29)], [("e", 1)]]
+    fed = {r: 0 for r in seqs}
+    steps = []
+    for n, items in enumerate(plan):
+        entries, end = [], []
+        for r, c in items:
+            entries.append({"id": r, "tokens": seqs[r][fed[r]:fed[r] + c], "want": list(range(c))})
+            fed[r] += c
+            if fed[r] == lens[r]:
+                end.append(r)
+        steps.append({"step": n, "entries": entries, "end": end})
+    assert fed == lens
+    out = tmp_path / f"out_{dtype}"
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+         "--out", str(out), "--max-tokens", "320"],
+        input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(len(plan))]
+    got = {r: [] for r in seqs}
+    for s in steps:
+        rows = torch.from_numpy(np.fromfile(out / f"{s['step']}.f32", dtype="<f4").reshape(-1, V))
+        o = 0
+        for e in s["entries"]:
+            got[e["id"]].append(rows[o:o + len(e["want"])])
+            o += len(e["want"])
+        assert o == rows.shape[0]
+    for r in seqs:
+        assert_close(torch.cat(got[r]), refs[r], dtype, r)
