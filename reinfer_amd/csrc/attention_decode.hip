@@ -119,6 +119,7 @@ flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restri
     const bool biased = MOD && mod.r1 != nullptr;
     const float r1h = (biased && r < G) ? mod.r1[kvh * G + r] : 0.f;
     const float r2h = (biased && r < G) ? mod.r2[kvh * G + r] : 0.f;
+    const float inv_cap = (MOD && mod.softcap > 0.f) ? 1.f / mod.softcap : 0.f;
 
     const int k_begin = cut.base + ci * cut.chunk;
     const int k_end = min(k_begin + cut.chunk, p + 1);
@@ -185,7 +186,7 @@ flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restri
           const int key = k0 + tt * 16 + 4 * g + i;
           float v = -INFINITY;
           if (key <= p && key >= lo) {
-            if (MOD) v = ra_mod_score(s[tt][i] * scale, mod.softcap, biased, r1h, r2h, p - key) * 1.4426950408889634f;
+            if (MOD) v = ra_mod_score_fast(s[tt][i] * scale, mod.softcap, inv_cap, biased, r1h, r2h, p - key) * 1.4426950408889634f;
             else v = s[tt][i] * scale_log2;
           }
           s[tt][i] = v;

@@ -117,6 +117,7 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
   bool q_live[NC];
   bf16x8_t qreg[NC][NDT];
   const bool biased = MOD && mod.r1 != nullptr;
+  const float inv_cap = (MOD && mod.softcap > 0.f) ? 1.f / mod.softcap : 0.f;
   float r1h[NC], r2h[NC];               // the distance term's two numbers of each column tile's head
 #pragma unroll
   for (int j = 0; j < NC; ++j) {
@@ -307,7 +308,8 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               const int key = kh + ks * 16 + 4 * g + i;
-              s[ks][j][i] = ra_mod_score(s[ks][j][i] * mod_scale, mod.softcap, biased, r1h[j], r2h[j], max(q_pos - key, 0));
+              s[ks][j][i] = ra_mod_score_fast(s[ks][j][i] * mod_scale, mod.softcap, inv_cap, biased, r1h[j], r2h[j],
+                                              max(q_pos - key, 0));
             }
         }
       }

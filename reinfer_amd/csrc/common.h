@@ -98,6 +98,17 @@ __device__ __forceinline__ float ra_mod_score(float s, float softcap, bool biase
   if (biased) s -= r1 * logf(1.f + r2 * (float)dist);
   return s;
 }
+// The same through the hardware's exponential, logarithm and reciprocal (an ulp or two each), for the kernels whose
+// operands are bfloat16: tanh(x) = 1 - 2 / (1 + e^(2x)), the argument bounded so that e^(2x) stays finite.
+__device__ __forceinline__ float ra_mod_score_fast(float s, float softcap, float inv_softcap, bool biased, float r1,
+                                                   float r2, int dist) {
+  if (softcap > 0.f) {
+    const float x = fminf(fmaxf(s * inv_softcap, -15.f), 15.f);
+    s = softcap * (1.f - __fdividef(2.f, 1.f + __expf(2.f * x)));
+  }
+  if (biased) s -= r1 * 0.6931471805599453f * __log2f(fmaf(r2, (float)dist, 1.f));
+  return s;
+}
 
 // ---- cache layout -----------------------------------------------------------
 // A block of the cache holds block_size (a multiple of 16) slots of one KV head

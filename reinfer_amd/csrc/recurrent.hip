@@ -169,9 +169,9 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
       if (kq_t[j] < n && kq_e[j]) {
         fk[j] = to_f32(kg[row0 + kq_g[j]]);
         fq[j] = to_f32(qg[row0 + kq_g[j]]) * p.q_scale;
-        if (DECAY) {
-          fk[j] = fk[j] / (1.f + expf(-fk[j]));
-          fq[j] = fq[j] / (1.f + expf(-fq[j]));
+        if (DECAY) {                                   // silu through the hardware's exponential and reciprocal
+          fk[j] = __fdividef(fk[j], 1.f + __expf(-fk[j]));
+          fq[j] = __fdividef(fq[j], 1.f + __expf(-fq[j]));
         }
       }
       if (WKV) {                                     // the decay exp(-exp(z + w0)), float from its pre-activation on
@@ -183,7 +183,7 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
 #pragma unroll
     for (int j = 0; j < SCAN_V_REGS; ++j) {
       fv[j] = v_t[j] < n ? to_f32(vg[row0 + v_g[j]]) : 0.f;
-      if (DECAY) fv[j] = fv[j] / (1.f + expf(-fv[j]));
+      if (DECAY) fv[j] = __fdividef(fv[j], 1.f + __expf(-fv[j]));
     }
     fg = (NG && g_t < n) ? p.gates[(size_t)t0 * NG * H + g_g] : 0.f;
   };
@@ -510,6 +510,50 @@ __global__ void head_norm_gate_kernel(const float* __restrict__ read, const floa
   }
 }
 
+// The same for heads wider than a wave can walk quickly (one "head" as wide as all read-outs together): a workgroup a
+// (token, head), every thread up to HNG_CHUNKS runs of eight neighbouring elements in registers, 16-byte accesses.
+#define HNG_CHUNKS 4
+template <typename TA>
+__global__ void head_norm_gate_wide_kernel(const float* __restrict__ read, const float* __restrict__ weight,
+                                           int w_head_stride, const TA* __restrict__ gate, int ldg, int silu, float eps,
+                                           int H, int dv, TA* __restrict__ out) {
+  __shared__ float red[17];
+  const long t = blockIdx.x / H;
+  const int h = blockIdx.x % H;
+  const float* x = read + (size_t)t * H * dv + (size_t)h * dv;
+  const TA* g = gate + (size_t)t * ldg + (size_t)h * dv;
+  const float* wt = weight + (size_t)h * w_head_stride;
+  TA* o = out + (size_t)t * H * dv + (size_t)h * dv;
+  float a[HNG_CHUNKS][8], w[HNG_CHUNKS][8], z[HNG_CHUNKS][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int r = 0; r < HNG_CHUNKS; ++r) {
+    const int c = (threadIdx.x + r * blockDim.x) * 8;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) a[r][e] = 0.f;
+    if (c >= dv) continue;
+    Vec8<float>::load(x + c, a[r]);
+    Vec8<float>::load(wt + c, w[r]);
+    Vec8<TA>::load(g + c, z[r]);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += a[r][e] * a[r][e];
+  }
+  const float total = block_sum(ss, red);
+  const float rstd = 1.f / sqrtf(total / (float)dv + eps);
+#pragma unroll
+  for (int r = 0; r < HNG_CHUNKS; ++r) {
+    const int c = (threadIdx.x + r * blockDim.x) * 8;
+    if (c >= dv) continue;
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float s = 1.f / (1.f + expf(-z[r][e]));
+      v[e] = a[r][e] * rstd * w[r][e] * (silu ? z[r][e] * s : s);
+    }
+    Vec8<TA>::store(o + c, v);
+  }
+}
+
 // ---------------------------------------------------------------------------
 // y[t, :] = (1 / n) sum_i x_i[t, :] / rms(x_i[t, :]) * w_i;  out = y, or resid += scale * y. One workgroup a row.
 // ---------------------------------------------------------------------------
@@ -775,6 +819,22 @@ extern "C" int ra_head_norm_gate(const float* read, const float* weight, int per
   const long units = (long)n_tokens * heads;
   const unsigned blocks = (unsigned)((units + 3) / 4);
   const int ws = per_head_weight ? value_dim : 0;
+  const int es = act_dtype == RA_F32 ? 4 : 2;
+  if (value_dim >= 512 && value_dim % 8 == 0 && value_dim <= 8 * HNG_CHUNKS * 1024 && units <= 0x7fffffffL &&
+      ((uintptr_t)read % 16) == 0 && ((uintptr_t)weight % 16) == 0 && ((uintptr_t)gate % 16) == 0 &&
+      ((long)ldg * es) % 16 == 0 && ((uintptr_t)out % 16) == 0 && (act_dtype == RA_F32 || act_dtype == RA_BF16)) {
+    int threads = (value_dim / 8 + RA_WAVE - 1) / RA_WAVE * RA_WAVE;
+    if (threads > 1024) threads = 1024;
+    if (act_dtype == RA_F32)
+      head_norm_gate_wide_kernel<float><<<(unsigned)units, threads, 0, stream>>>(read, weight, ws, (const float*)gate, ldg,
+                                                                                 silu, eps, heads, value_dim, (float*)out);
+    else
+      head_norm_gate_wide_kernel<bf16_t><<<(unsigned)units, threads, 0, stream>>>(read, weight, ws, (const bf16_t*)gate,
+                                                                                  ldg, silu, eps, heads, value_dim,
+                                                                                  (bf16_t*)out);
+    RA_LAUNCH_CHECK("head_norm_gate");
+    return 0;
+  }
   if (act_dtype == RA_F32)
     head_norm_gate_kernel<float><<<blocks, 4 * RA_WAVE, 0, stream>>>(read, weight, ws, (const float*)gate, ldg, silu,
                                                                      eps, heads, value_dim, (float*)out, units);

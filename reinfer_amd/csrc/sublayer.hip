@@ -74,6 +74,55 @@ __global__ void sum_norm_add_kernel(SumInputs in, const float* __restrict__ weig
   }
 }
 
+// The same with rows whose width is a multiple of 8 and at most 8 * SNA_CHUNKS * 1024: a thread holds up to SNA_CHUNKS
+// runs of eight neighbouring elements in registers, everything it reads (the inputs, the stream, the weight) is
+// asked for in one trip through 16-byte accesses, and nothing is read twice.
+#define SNA_CHUNKS 4
+template <typename TX, typename TO, int N>
+__global__ void sum_norm_add_vec_kernel(SumInputs in, const float* __restrict__ weight, int weight_stride, int normed,
+                                        float eps, int h, float* __restrict__ resid, TO* __restrict__ copy) {
+  __shared__ float red[17];
+  const size_t row = (size_t)blockIdx.x * h;
+  float y[SNA_CHUNKS][8], add[SNA_CHUNKS][8], w[SNA_CHUNKS][8];
+  bool live[SNA_CHUNKS];
+  float ss = 0.f;
+#pragma unroll
+  for (int r = 0; r < SNA_CHUNKS; ++r) {
+    const int c = (threadIdx.x + r * blockDim.x) * 8;
+    live[r] = c < h;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { y[r][e] = 0.f; add[r][e] = 0.f; w[r][e] = 1.f; }
+    if (!live[r]) continue;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      float v[8];
+      Vec8<TX>::load((const TX*)in.x[i] + row + c, v);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) y[r][e] += in.s[i] * v[e];
+    }
+    if (resid) Vec8<float>::load(resid + row + c, add[r]);
+    if (normed && weight_stride) Vec8<float>::load(weight + c, w[r]);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += y[r][e] * y[r][e];
+  }
+  float rstd = 1.f;
+  if (normed) {
+    const float total = block_sum(ss, red);
+    rstd = 1.f / sqrtf(total / (float)h + eps);
+    if (!weight_stride) rstd *= weight[0];
+  }
+#pragma unroll
+  for (int r = 0; r < SNA_CHUNKS; ++r) {
+    if (!live[r]) continue;
+    const int c = (threadIdx.x + r * blockDim.x) * 8;
+    float o[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (normed ? y[r][e] * rstd * w[r][e] : y[r][e]) + add[r][e];
+    if (resid) Vec8<float>::store(resid + row + c, o);
+    if (copy) Vec8<TO>::store(copy + row + c, o);
+  }
+}
+
 // One workgroup a (row, span): blockIdx.y picks the span.
 struct NormSpans {
   int col0[2], width[2], count[2];
@@ -94,6 +143,41 @@ __global__ void span_rmsnorm_kernel(TA* __restrict__ x, long ld, NormSpans sp, f
   const float rstd = 1.f / sqrtf(total / (float)sp.count[k] + eps);
   const float* w = sp.w[k];
   for (int e = threadIdx.x; e < n; e += blockDim.x) v[e] = from_f32<TA>(to_f32(v[e]) * rstd * w[e]);
+}
+
+// The same for runs that start and end on multiples of 8 columns and are at most 8 * SNA_CHUNKS * 1024 wide: a run in
+// registers, 16-byte accesses, one trip to memory.
+template <typename TA>
+__global__ void span_rmsnorm_vec_kernel(TA* __restrict__ x, long ld, NormSpans sp, float eps) {
+  __shared__ float red[17];
+  const int k = blockIdx.y;
+  TA* v = x + (size_t)blockIdx.x * ld + sp.col0[k];
+  const int n = sp.width[k];
+  const float* wt = sp.w[k];
+  float a[SNA_CHUNKS][8], w[SNA_CHUNKS][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int r = 0; r < SNA_CHUNKS; ++r) {
+    const int c = (threadIdx.x + r * blockDim.x) * 8;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) a[r][e] = 0.f;
+    if (c >= n) continue;
+    Vec8<TA>::load(v + c, a[r]);
+    Vec8<float>::load(wt + c, w[r]);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += a[r][e] * a[r][e];
+  }
+  const float total = block_sum(ss, red);
+  const float rstd = 1.f / sqrtf(total / (float)sp.count[k] + eps);
+#pragma unroll
+  for (int r = 0; r < SNA_CHUNKS; ++r) {
+    const int c = (threadIdx.x + r * blockDim.x) * 8;
+    if (c >= n) continue;
+    float o[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = a[r][e] * rstd * w[r][e];
+    Vec8<TA>::store(v + c, o);
+  }
 }
 
 // One thread a (token, head, pair).
@@ -169,10 +253,24 @@ extern "C" int ra_sum_norm_add(const void* const* xs, const float* scales, int n
     in.x[i] = i < n ? xs[i] : nullptr;
     in.s[i] = i < n ? scales[i] : 0.f;
   }
-  const int threads = hidden >= 2048 ? 512 : 256;
-#define RA_SNA(TX, TO, N)                                                                                      \
-  sum_norm_add_kernel<TX, TO, N><<<n_tokens, threads, 0, stream>>>(in, weight, weight_stride, normed, eps, hidden, \
-                                                                   resid, (TO*)copy)
+  int threads = hidden >= 2048 ? 512 : 256;
+  // rows of whole 16-byte pieces in every operand: the form that keeps a row in registers
+  bool vec = hidden % 8 == 0 && hidden <= 8 * SNA_CHUNKS * 1024 && ((uintptr_t)resid % 16) == 0 &&
+             ((uintptr_t)copy % 16) == 0 && (!normed || weight_stride == 0 || ((uintptr_t)weight % 16) == 0);
+  for (int i = 0; i < n; ++i) vec = vec && ((uintptr_t)xs[i] % 16) == 0;
+  if (vec) {
+    threads = (hidden / 8 + RA_WAVE - 1) / RA_WAVE * RA_WAVE;
+    if (threads > 1024) threads = 1024;
+  }
+#define RA_SNA(TX, TO, N)                                                                                          \
+  do {                                                                                                             \
+    if (vec)                                                                                                       \
+      sum_norm_add_vec_kernel<TX, TO, N><<<n_tokens, threads, 0, stream>>>(in, weight, weight_stride, normed, eps, \
+                                                                           hidden, resid, (TO*)copy);              \
+    else                                                                                                           \
+      sum_norm_add_kernel<TX, TO, N><<<n_tokens, threads, 0, stream>>>(in, weight, weight_stride, normed, eps,     \
+                                                                       hidden, resid, (TO*)copy);                  \
+  } while (0)
 #define RA_SNA_N(TX, TO)                \
   do {                                  \
     if (n == 1) RA_SNA(TX, TO, 1);      \
@@ -207,9 +305,22 @@ extern "C" int ra_span_rmsnorm(void* x, int act_dtype, long ld, int n_tokens, in
   }
   RA_CHECK(n_tokens <= 0x7fffffff / 1, "span_rmsnorm: too many rows");
   const dim3 grid(n_tokens, n_spans);
-  if (act_dtype == RA_F32) span_rmsnorm_kernel<float><<<grid, 256, 0, stream>>>((float*)x, ld, sp, eps);
-  else if (act_dtype == RA_BF16) span_rmsnorm_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)x, ld, sp, eps);
-  else return ra_fail("span_rmsnorm: unknown dtype tag %d", act_dtype);
+  const int es = act_dtype == RA_F32 ? 4 : 2;
+  bool vec = ((uintptr_t)x % 16) == 0 && (ld * es) % 16 == 0;
+  int widest = 0;
+  for (int k = 0; k < n_spans; ++k) {
+    vec = vec && col0[k] % 8 == 0 && width[k] % 8 == 0 && width[k] <= 8 * SNA_CHUNKS * 1024 && ((uintptr_t)w[k] % 16) == 0;
+    widest = width[k] > widest ? width[k] : widest;
+  }
+  int threads = (widest / 8 + RA_WAVE - 1) / RA_WAVE * RA_WAVE;
+  if (threads > 1024) threads = 1024;
+  if (act_dtype == RA_F32) {
+    if (vec) span_rmsnorm_vec_kernel<float><<<grid, threads, 0, stream>>>((float*)x, ld, sp, eps);
+    else span_rmsnorm_kernel<float><<<grid, 256, 0, stream>>>((float*)x, ld, sp, eps);
+  } else if (act_dtype == RA_BF16) {
+    if (vec) span_rmsnorm_vec_kernel<bf16_t><<<grid, threads, 0, stream>>>((bf16_t*)x, ld, sp, eps);
+    else span_rmsnorm_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)x, ld, sp, eps);
+  } else return ra_fail("span_rmsnorm: unknown dtype tag %d", act_dtype);
   RA_LAUNCH_CHECK("span_rmsnorm");
   return 0;
 }

@@ -316,3 +316,22 @@ def test_experts_from_the_table_and_the_bounded_activation():
             close(got, want, 2e-6 if dtype == torch.float32 else 2 ** -8, (I, group))
     with pytest.raises(ValueError):
         ops.silu_mul(gu.to(DEV), got, 0, act="swish_bounded")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,dv", [(1, 4096), (1, 520), (3, 512), (1, 96), (2, 9000)])
+def test_head_norm_gate_over_wide_heads(dtype, H, dv):
+    """One norm over all read-outs of a row (a single head as wide as all of them), and heads wide enough for the
+    form that gives a workgroup to each."""
+    ops, ref = kernels.current(), KernelDouble()
+    g = torch.Generator().manual_seed(dv)
+    T, n = 5, H * dv
+    read = torch.randn(T, n, generator=g) * 3
+    weight = torch.rand(n, generator=g) + 0.5
+    gate = torch.randn(T, n + 16, generator=g).to(dtype)
+    for kind in ("sigmoid", "silu"):
+        want = torch.empty(T, n, dtype=dtype)
+        ref.head_norm_gate(read, weight, True, gate, kind, 1e-5, H, dv, want)
+        got = torch.empty(T, n, dtype=dtype, device=DEV)
+        ops.head_norm_gate(read.to(DEV), weight.to(DEV), True, gate.to(DEV), kind, 1e-5, H, dv, got)
+        close(got, want, 2e-6 if dtype == torch.float32 else 2 ** -8, (H, dv, kind))
