@@ -74,20 +74,21 @@ __global__ void sum_norm_add_kernel(SumInputs in, const float* __restrict__ weig
   }
 }
 
-// The same with rows whose width is a multiple of 8 and at most 8 * SNA_CHUNKS * 1024: a thread holds up to SNA_CHUNKS
+// The same with rows whose width is a multiple of 8 and at most 8 * SNA_CHUNKS * 1024: a thread holds CH (1, 2 or 4)
 // runs of eight neighbouring elements in registers, everything it reads (the inputs, the stream, the weight) is
-// asked for in one trip through 16-byte accesses, and nothing is read twice.
+// asked for in one trip through 16-byte accesses, and nothing is read twice. (CH is a template parameter so that a
+// row of 2,048 or 4,096 costs the registers of one or two runs, not of four, and more workgroups share a CU.)
 #define SNA_CHUNKS 4
-template <typename TX, typename TO, int N>
+template <typename TX, typename TO, int N, int CH>
 __global__ void sum_norm_add_vec_kernel(SumInputs in, const float* __restrict__ weight, int weight_stride, int normed,
                                         float eps, int h, float* __restrict__ resid, TO* __restrict__ copy) {
   __shared__ float red[17];
   const size_t row = (size_t)blockIdx.x * h;
-  float y[SNA_CHUNKS][8], add[SNA_CHUNKS][8], w[SNA_CHUNKS][8];
-  bool live[SNA_CHUNKS];
+  float y[CH][8], add[CH][8], w[CH][8];
+  bool live[CH];
   float ss = 0.f;
 #pragma unroll
-  for (int r = 0; r < SNA_CHUNKS; ++r) {
+  for (int r = 0; r < CH; ++r) {
     const int c = (threadIdx.x + r * blockDim.x) * 8;
     live[r] = c < h;
 #pragma unroll
@@ -112,7 +113,7 @@ __global__ void sum_norm_add_vec_kernel(SumInputs in, const float* __restrict__ 
     if (!weight_stride) rstd *= weight[0];
   }
 #pragma unroll
-  for (int r = 0; r < SNA_CHUNKS; ++r) {
+  for (int r = 0; r < CH; ++r) {
     if (!live[r]) continue;
     const int c = (threadIdx.x + r * blockDim.x) * 8;
     float o[8];
@@ -258,15 +259,21 @@ extern "C" int ra_sum_norm_add(const void* const* xs, const float* scales, int n
   bool vec = hidden % 8 == 0 && hidden <= 8 * SNA_CHUNKS * 1024 && ((uintptr_t)resid % 16) == 0 &&
              ((uintptr_t)copy % 16) == 0 && (!normed || weight_stride == 0 || ((uintptr_t)weight % 16) == 0);
   for (int i = 0; i < n; ++i) vec = vec && ((uintptr_t)xs[i] % 16) == 0;
+  int chunks = 1;
   if (vec) {
-    threads = (hidden / 8 + RA_WAVE - 1) / RA_WAVE * RA_WAVE;
-    if (threads > 1024) threads = 1024;
+    // rows up to 2,048 wide: one run a thread; from there workgroups of 256 threads with two or four runs each, and
+    // beyond 8,192 more threads
+    chunks = hidden <= 2048 ? 1 : hidden <= 4096 ? 2 : 4;
+    threads = (hidden / (8 * chunks) + RA_WAVE - 1) / RA_WAVE * RA_WAVE;
   }
+#define RA_SNA_VEC(TX, TO, N, CH)                                                                                      \
+  sum_norm_add_vec_kernel<TX, TO, N, CH><<<n_tokens, threads, 0, stream>>>(in, weight, weight_stride, normed, eps,     \
+                                                                           hidden, resid, (TO*)copy)
 #define RA_SNA(TX, TO, N)                                                                                          \
   do {                                                                                                             \
-    if (vec)                                                                                                       \
-      sum_norm_add_vec_kernel<TX, TO, N><<<n_tokens, threads, 0, stream>>>(in, weight, weight_stride, normed, eps, \
-                                                                           hidden, resid, (TO*)copy);              \
+    if (vec && chunks == 1) RA_SNA_VEC(TX, TO, N, 1);                                                              \
+    else if (vec && chunks == 2) RA_SNA_VEC(TX, TO, N, 2);                                                         \
+    else if (vec) RA_SNA_VEC(TX, TO, N, 4);                                                                        \
     else                                                                                                           \
       sum_norm_add_kernel<TX, TO, N><<<n_tokens, threads, 0, stream>>>(in, weight, weight_stride, normed, eps,     \
                                                                        hidden, resid, (TO*)copy);                  \
@@ -286,6 +293,7 @@ extern "C" int ra_sum_norm_add(const void* const* xs, const float* scales, int n
   else return ra_fail("sum_norm_add: unknown dtype tags %d, %d", in_dtype, copy_dtype);
 #undef RA_SNA_N
 #undef RA_SNA
+#undef RA_SNA_VEC
   RA_LAUNCH_CHECK("sum_norm_add");
   return 0;
 }

@@ -238,9 +238,11 @@ class HipKernels:
         """
         lib = library.load()
         mod = self._score_mod(softcap, distance, num_heads, q.device)
+        # handed on only where there is a change, so that the kernels' callers of old need not know of it
+        changed = {"mod": mod} if (mod[0] > 0.0 or mod[1] is not None) else {}
         if q.dtype != torch.bfloat16:
             return self.attention_plain(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
-                                        head_dim, scale, window, group, mod=mod)
+                                        head_dim, scale, window, group, **changed)
         bs = kcache.shape[2] * 16
         tile = lib.ra_attention_prefill_tile(num_heads, num_kv_heads, head_dim)
         # query tiles that give every CU one workgroup
@@ -265,24 +267,24 @@ class HipKernels:
             with torch.cuda.stream(side):           # its scratch comes from, and goes back to, the side stream's pool
                 self.attention_decode(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
                                       head_dim, scale, window, group, plan["decode_list"], plan["n_decode"],
-                                      plan["decode_max_ctx"], mod=mod)
+                                      plan["decode_max_ctx"], **changed)
         elif plan["n_decode"]:
             if dec_ok:
                 self.attention_decode(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
                                       head_dim, scale, window, group, plan["decode_list"], plan["n_decode"],
-                                      plan["decode_max_ctx"], mod=mod)
+                                      plan["decode_max_ctx"], **changed)
             else:
                 self.attention_plain(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
-                                     head_dim, scale, window, group, plan["decode_list"], plan["n_decode"], mod=mod)
+                                     head_dim, scale, window, group, plan["decode_list"], plan["n_decode"], **changed)
         if plan["n_tiles"]:
             if pre_ok:
                 self.attention_prefill(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
                                        head_dim, scale, window, group, plan["tiles"], plan["n_tiles"],
                                        plan.get("ranges"), plan.get("merge"), plan.get("n_merge", 0),
-                                       plan.get("n_slots", 0), mod=mod)
+                                       plan.get("n_slots", 0), **changed)
             else:
                 self.attention_plain(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
-                                     head_dim, scale, window, group, plan["prefill_list"], plan["n_prefill"], mod=mod)
+                                     head_dim, scale, window, group, plan["prefill_list"], plan["n_prefill"], **changed)
         if side is not None:
             torch.cuda.current_stream().wait_stream(side)
 

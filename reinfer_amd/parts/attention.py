@@ -121,6 +121,10 @@ class GroupedQueryAttention:
             # the further options run as kernels of their own around the attention: no norm rides on this
             # mixer's products, and its result goes back to the caller
             self.adds_in_place = self.takes_row_scaled = self.emits_for_norm = False
+        if (key_dim != D or value_dim != D) and (spec.qk_norm or spec.bias) and not self.extended:
+            raise ValueError(f"attention: heads of {key_dim} / {value_dim} are laid out with zeros behind them, which a "
+                             "head norm or a bias takes only on the path of the further options: without those, head "
+                             "sizes go in steps of 16")
         if spec.qk_norm and spec.qk_norm_whole:
             raise ValueError("attention: q and k are normed per head or over their whole projection, not both")
 
