@@ -498,7 +498,7 @@ def _gibavik_raw(width, vocab, pattern, attn, right, dense_ff, moe):
             "scale": 128 ** -0.5, "softcap": 30.0, "vdim": 128}
     memory = {"decay": [1.0 - 2.0 ** -(2 + 6 * h / max(1, right - 1)) for h in range(right)], "dim": 128, "heads": right,
               "vdim": 128}
-    pair = {"left": left, "left_scale": 0.6, "right": memory, "right_scale": 0.9}
+    pair = {"left": left, "left_scale": 0.5, "right": memory, "right_scale": 1.25}
     dense = {"ff": dense_ff, "kind": "dense", "limit": 7.0}
     experts = {"expert": {"ff": moe[2]}, "kind": "moe", "router": {"experts": moe[0], "top": moe[1]}}
     layers = []
@@ -510,8 +510,8 @@ def _gibavik_raw(width, vocab, pattern, attn, right, dense_ff, moe):
             layers.append({"type": "attention", "mixer": dict(full, kv_from=j), "mlp": experts})
         else:
             layers.append({"type": "attention", "mixer": full, "mlp": dense if c == "A" else experts})
-    return {"architecture": "Gibavik", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "embedding": {"scale": 12.0},
-            "logit_softcap": 15.0, "layers": layers}
+    return {"architecture": "Gibavik", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "embedding": {"scale": 6.0},
+            "logit_softcap": 25.0, "layers": layers}
 
 
 # (name, Gibavik configuration, its Kobolix twin, vocabulary, "kobolix"): as many layers, the same width, the same

@@ -33,7 +33,7 @@ def _attn(heads, kv, dim, vdim, scale=None, kv_from=None, window=None):
     return m
 
 
-def _left(heads, kv, dim, vdim, window, dims, base=10000.0, cap=20.0, scale=None):
+def _left(heads, kv, dim, vdim, window, dims, base=10000.0, cap=25.0, scale=None):
     m = {"dim": dim, "heads": heads, "kv_heads": kv, "scale": dim ** -0.5 if scale is None else scale, "vdim": vdim}
     if window:
         m["mask"] = {"size": window}

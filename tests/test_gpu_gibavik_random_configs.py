@@ -45,11 +45,11 @@ def draw_config(rng: random.Random, wide: bool = False) -> dict:
         m = {"dim": dim, "heads": H, "kv_heads": G,
              "vdim": rng.choice([4, 8, 16, 20, 32, 56] if not wide else [32, 64, 96, 128])}
         if rng.random() < 0.85:
-            m["mask"] = {"size": rng.choice([1, 2, 5, 16, 17, 33, 64] if not wide else [16, 100, 136, 257])}
+            m["mask"] = {"size": rng.choice([1, 2, 5, 16, 17, 33, 64] if not wide else [16, 100, 150, 257])}
         if rng.random() < 0.85:
-            m["rot"] = {"base": rng.choice([100.0, 10000.0, 250000.0]), "dims": rng.choice([d for d in (2, 4, 8, 16, 32, 64, dim) if d <= dim and d % 2 == 0])}
+            m["rot"] = {"base": rng.choice([100.0, 10000.0, 500000.0]), "dims": rng.choice([d for d in (2, 4, 8, 16, 32, 64, dim) if d <= dim and d % 2 == 0])}
         if rng.random() < 0.8:
-            m["softcap"] = rng.choice([2.0, 20.0, 50.0])
+            m["softcap"] = rng.choice([2.0, 25.0, 50.0])
         if rng.random() < 0.8:
             m["scale"] = rng.choice([0.1, 0.25, 0.5])
         return m
@@ -80,16 +80,16 @@ def draw_config(rng: random.Random, wide: bool = False) -> dict:
         elif rng.random() < 0.5:
             pair = {"left": left(), "right": right()}
             if rng.random() < 0.8:
-                pair["left_scale"], pair["right_scale"] = rng.choice([0.3, 0.6, 1.0]), rng.choice([0.5, 0.9, 1.4])
+                pair["left_scale"], pair["right_scale"] = rng.choice([0.3, 0.7, 1.0]), rng.choice([0.5, 0.8, 1.4])
             layers.append({"type": "parallel", "mixer": pair, "mlp": mlp()})
         else:
             layers.append({"type": "attention", "mixer": full(), "mlp": mlp()})
     raw = {"architecture": "Gibavik", "vocab": rng.choice([50, 131, 400]), "width": width,
            "norm": {"eps": rng.choice([1e-6, 1e-5])}, "layers": layers}
     if rng.random() < 0.8:
-        raw["embedding"] = {"scale": rng.choice([1.0, 3.0, 12.0])}
+        raw["embedding"] = {"scale": rng.choice([1.0, 3.0, 9.0])}
     if rng.random() < 0.8:
-        raw["logit_softcap"] = rng.choice([5.0, 15.0, 30.0])
+        raw["logit_softcap"] = rng.choice([5.0, 18.0, 30.0])
     return raw
 
 
