@@ -473,22 +473,25 @@ def test_greedy_generation_gpu(tmp_path_factory, which, dtype):
 
 
 @pytest.mark.gpu
-def test_captured_decode_steps_gpu(tmp_path_factory):
+@pytest.mark.parametrize("which,dtype", [("A", "float32"), ("C", "bfloat16")])
+def test_captured_decode_steps_gpu(tmp_path_factory, which, dtype):
     """Decode steps replay captured graphs: the same logits as a runner without graphs, over several replays
-    with eager prompt steps between them, state slots and blocks changing hands meanwhile."""
-    folder = make_folder(tmp_path_factory.getbasetemp(), "A", "float32")
-    seqs = {r: random_tokens(n, vocab("A"), 500 + i) for i, (r, n) in enumerate((("a", 40), ("b", 25), ("c", 31)))}
+    with eager prompt steps between them, state slots and blocks changing hands meanwhile. (bfloat16: a captured
+    step cuts a token's keys into chunks by its context bucket, not by the step's longest context, so the two
+    runners add the same terms in another order.)"""
+    folder = make_folder(tmp_path_factory.getbasetemp(), which, dtype)
+    seqs = {r: random_tokens(n, vocab(which), 500 + i) for i, (r, n) in enumerate((("a", 40), ("b", 25), ("c", 31)))}
     plan = [[("a", 10), ("b", 5)]] + [[("a", 1), ("b", 1)]] * 6 + [[("c", 9)]] + [[("a", 1), ("b", 1), ("c", 1)]] * 8 \
         + [[("a", 16), ("b", 6), ("c", 14)]]
     outs = []
     for graphs in (True, False):
-        runner = runner_for(folder, "cuda:0", "float32", max_tokens=256, use_graphs=graphs)
+        runner = runner_for(folder, "cuda:0", dtype, max_tokens=256, use_graphs=graphs)
         outs.append(run_plan(runner, seqs, plan))
         if graphs:
             assert runner.graphs is not None and runner.graphs.replays >= 14
     for r, toks in seqs.items():
-        assert rel_err(outs[0][r], outs[1][r]) < 1e-6, r
-        assert rel_err(outs[0][r], reference(folder, toks)) < TOL["float32"], r
+        assert rel_err(outs[0][r], outs[1][r]) < (1e-6 if dtype == "float32" else 2e-2), r
+        assert_close(outs[0][r], reference(folder, toks), dtype, r)
 
 
 def test_command_line_init_writes_a_loadable_folder(tmp_path):
